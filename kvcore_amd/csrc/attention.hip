@@ -6,7 +6,8 @@
 // tile: each lane scores one key (a float32 dot product over the head in index
 // order), the tile is folded into a running softmax (float32 max, sum and output
 // accumulators), then the lanes split the head's elements to add p_j * V_j in key
-// order.  K pages are [kv head, page_size, d], V pages [kv head, d, page_size].  What a token computes depends on its position, window and cache content
+// order.  K pages are [kv head, page_size, d], V pages [kv head, dv, page_size]: keys of d
+// elements and values of dv, which need not be equal.  What a token computes depends on its position, window and cache content
 // only: not on the batch it is in nor on how its request was cut into steps.
 
 #include <hip/hip_runtime.h>
@@ -44,7 +45,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     T* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
-    const int32_t* __restrict__ slots, int nh, int nkv, int d, int page_size, int num_pages,
+    const int32_t* __restrict__ slots, int nh, int nkv, int d, int dv, int page_size, int num_pages,
     float scale, int window) {
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
   __shared__ float p_s[kWavesPerBlock][kWave];
@@ -57,12 +58,12 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   const int h_raw = blockIdx.y * kWavesPerBlock + wave;
   const bool head_live = h_raw < nh;
   const int h = head_live ? h_raw : nh - 1;
-  T* o = out + (static_cast<int64_t>(t) * nh + h) * d;
+  T* o = out + (static_cast<int64_t>(t) * nh + h) * dv;
 
   const int req = token_req[t];
   if (req < 0) {  // padding token: the whole block takes this branch
     if (head_live)
-      for (int i = lane; i < d; i += kWave) o[i] = from_float<T>(0.f);
+      for (int i = lane; i < dv; i += kWave) o[i] = from_float<T>(0.f);
     return;
   }
   const int pos = positions[t];
@@ -82,6 +83,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   constexpr int VN = Vec16<T>::N;
   const int64_t head_off = static_cast<int64_t>(hk) * page_size * d;
   const int64_t page_elems = static_cast<int64_t>(nkv) * page_size * d;
+  const int64_t v_head_off = static_cast<int64_t>(hk) * page_size * dv;
+  const int64_t v_page_elems = static_cast<int64_t>(nkv) * page_size * dv;
 
   for (int tile = first; tile <= pos; tile += kWave) {
     const int key = tile + lane;
@@ -93,13 +96,17 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
       if (page > 0 && page < num_pages) {
         off = static_cast<int64_t>(page) * page_elems + head_off +
               static_cast<int64_t>(key % page_size) * d;
-        voff = static_cast<int64_t>(page) * page_elems + head_off + key % page_size;
+        voff = static_cast<int64_t>(page) * v_page_elems + v_head_off + key % page_size;
         const T* kr = k_cache + off;
         float dot = 0.f;
-        for (int i = 0; i < d; i += VN) {
-          const Vec16<T> kv = *reinterpret_cast<const Vec16<T>*>(kr + i);
+        if (d % VN == 0) {
+          for (int i = 0; i < d; i += VN) {
+            const Vec16<T> kv = *reinterpret_cast<const Vec16<T>*>(kr + i);
 #pragma unroll
-          for (int e = 0; e < VN; ++e) dot = fmaf(q_s[wave][i + e], kv.get(e), dot);
+            for (int e = 0; e < VN; ++e) dot = fmaf(q_s[wave][i + e], kv.get(e), dot);
+          }
+        } else {  // a key size that 16-byte loads do not divide: element by element
+          for (int i = 0; i < d; ++i) dot = fmaf(q_s[wave][i], to_float(kr[i]), dot);
         }
         s = dot * scale;
       }
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
 #pragma unroll
       for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
         const int e = lane + i * kWave;
-        if (e < d) acc[i] = fmaf(pj, to_float(vr[static_cast<int64_t>(e) * page_size]), acc[i]);
+        if (e < dv) acc[i] = fmaf(pj, to_float(vr[static_cast<int64_t>(e) * page_size]), acc[i]);
       }
     }
   }
@@ -137,7 +144,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
 #pragma unroll
   for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
     const int e = lane + i * kWave;
-    if (e < d) o[e] = from_float<T>(acc[i] * inv);
+    if (e < dv) o[e] = from_float<T>(acc[i] * inv);
   }
 }
 
@@ -146,16 +153,18 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
 extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                                    const void* v_cache, const int32_t* table, int table_stride,
                                    const int32_t* positions, const int32_t* token_req,
-                                   const int32_t* slots, int T, int nh, int nkv, int d,
+                                   const int32_t* slots, int T, int nh, int nkv, int d, int dv,
                                    int page_size, int num_pages, float scale, int window,
                                    int dtype, kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || page_size <= 0 || num_pages <= 0 || table_stride <= 0)
     return kvc_fail("kvc_paged_attention: bad sizes");
   if (nh % nkv) return kvc_fail("kvc_paged_attention: heads must be a multiple of kv heads");
-  if (d <= 0 || d % 16 || d > kMaxHeadDim)
-    return kvc_fail("kvc_paged_attention: head size must be a multiple of 16, at most 256");
-  if (q_stride < static_cast<int64_t>(nh) * d || q_stride % 8)
-    return kvc_fail("kvc_paged_attention: q stride too small or not a multiple of 8");
+  if (d <= 0 || d > kMaxHeadDim)
+    return kvc_fail("kvc_paged_attention: head size must be positive, at most 256");
+  if (dv <= 0 || dv > kMaxHeadDim)
+    return kvc_fail("kvc_paged_attention: value size must be positive, at most 256");
+  if (q_stride < static_cast<int64_t>(nh) * d)
+    return kvc_fail("kvc_paged_attention: q stride too small");
   if (T == 0) return 0;
   const dim3 grid(T, (nh + kWavesPerBlock - 1) / kWavesPerBlock);
   KVC_DISPATCH_DTYPE(
@@ -164,6 +173,123 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(out),
                          static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                          static_cast<const Tp*>(v_cache), table, table_stride, positions,
-                         token_req, slots, nh, nkv, d, page_size, num_pages, scale, window));
+                         token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window));
   return kvc_check_launch("kvc_paged_attention");
+}
+
+// ------------------------------------- per-head norm, rotation and the K/V write in one
+// One block of four waves per token; a wave takes one head at a time.  A q or k head of d
+// elements is (optionally) divided by its root mean square, eps inside the root, and
+// multiplied by a gain shared by all heads; then its first rot_dim elements are rotated
+// (pairs (2j, 2j+1) when interleaved, (j, j + rot_dim/2) otherwise); all in float32, rounded
+// once on the way out.  q heads go back in place, k heads in place and to K[page, kv head,
+// offset, :]; the value heads of dv elements are copied to V[page, kv head, :, offset].
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
+    T* __restrict__ qkv, int64_t row_stride, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
+    int interleaved, const int32_t* __restrict__ kv_slot, int nh, int nkv, int d, int dv,
+    int page_size, int write_kv) {
+  __shared__ float head_s[4][kMaxHeadDim];
+  const int t = blockIdx.x;
+  const int slot = kv_slot[t];
+  if (slot == -2) return;  // padding token
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int half = rot_dim / 2;
+  T* row = qkv + static_cast<int64_t>(t) * row_stride;
+  const bool store_kv = write_kv && slot >= 0;
+  const int page = store_kv ? slot / page_size : 0;
+  const int off = store_kv ? slot - page * page_size : 0;
+  const float* cs = cos_tab + static_cast<int64_t>(t) * half;
+  const float* sn = sin_tab + static_cast<int64_t>(t) * half;
+
+  for (int head_base = 0; head_base < nh + nkv; head_base += 4) {  // every wave the same count
+    const bool live = head_base + wave < nh + nkv;
+    const int head = live ? head_base + wave : 0;
+    T* hp = row + static_cast<int64_t>(head) * d;
+    const float* gain = head < nh ? q_gain : k_gain;
+    float x[kMaxHeadDim / kWave];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+      const int e = lane + i * kWave;
+      x[i] = e < d ? to_float(hp[e]) : 0.f;
+      ss = fmaf(x[i], x[i], ss);
+    }
+    if (gain != nullptr) {
+      ss = wave_sum(ss);
+      const float inv = 1.f / sqrtf(ss / static_cast<float>(d) + eps);
+#pragma unroll
+      for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+        const int e = lane + i * kWave;
+        if (e < d) x[i] = x[i] * inv * gain[e];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+      const int e = lane + i * kWave;
+      if (e < d) head_s[wave][e] = x[i];
+    }
+    __syncthreads();
+    T* kc = nullptr;
+    if (live && head >= nh && store_kv)
+      kc = k_cache + ((static_cast<int64_t>(page) * nkv + (head - nh)) * page_size + off) * d;
+#pragma unroll
+    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+      const int e = lane + i * kWave;
+      if (e >= d || !live) continue;
+      float y = x[i];
+      if (e < rot_dim) {
+        int j, e0, e1;
+        if (interleaved) {
+          j = e >> 1; e0 = e & ~1; e1 = e0 + 1;
+        } else {
+          j = e < half ? e : e - half; e0 = j; e1 = j + half;
+        }
+        const float x0 = head_s[wave][e0], x1 = head_s[wave][e1];
+        y = (e == e0) ? rotate_first(x0, x1, cs[j], sn[j]) : rotate_second(x0, x1, cs[j], sn[j]);
+      }
+      const T r = from_float<T>(y);
+      hp[e] = r;
+      if (kc != nullptr) kc[e] = r;
+    }
+    __syncthreads();
+  }
+  if (!store_kv) return;
+  const T* vrow = row + static_cast<int64_t>(nh + nkv) * d;
+  const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * dv + off;
+  for (int w = threadIdx.x; w < nkv * dv; w += blockDim.x)
+    v_cache[v_base + static_cast<int64_t>(w) * page_size] = vrow[w];  // w = head * dv + i
+}
+
+}  // namespace
+
+extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache, void* v_cache,
+                                         const float* q_gain, const float* k_gain, float eps,
+                                         const float* cos_tab, const float* sin_tab, int rot_dim,
+                                         int interleaved, const int32_t* kv_slot, int T, int nh,
+                                         int nkv, int d, int dv, int page_size, int write_kv,
+                                         int dtype, kvc_stream stream) {
+  if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || dv <= 0 || page_size <= 0)
+    return kvc_fail("kvc_qk_norm_rope_kv_write: bad sizes");
+  if (d > kMaxHeadDim) return kvc_fail("kvc_qk_norm_rope_kv_write: head size above 256");
+  if (rot_dim < 0 || rot_dim > d || (rot_dim & 1))
+    return kvc_fail("kvc_qk_norm_rope_kv_write: rot_dim must be even and at most the head size");
+  if (row_stride < static_cast<int64_t>(nh + nkv) * d + static_cast<int64_t>(nkv) * dv)
+    return kvc_fail("kvc_qk_norm_rope_kv_write: rows too short for the heads");
+  if ((q_gain == nullptr) != (k_gain == nullptr))
+    return kvc_fail("kvc_qk_norm_rope_kv_write: gains for both q and k, or for neither");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(
+      dtype, Tp,
+      hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<Tp>, dim3(T), dim3(256), 0,
+                         reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
+                         static_cast<Tp*>(k_cache), static_cast<Tp*>(v_cache), q_gain, k_gain, eps,
+                         cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,
+                         write_kv));
+  return kvc_check_launch("kvc_qk_norm_rope_kv_write");
 }

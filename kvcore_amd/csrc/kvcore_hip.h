@@ -112,12 +112,82 @@ int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_
 
 // Attention of every token over its request's cache: token t at position p sees keys
 // max(0, p - window + 1) .. p (window <= 0: all), read through the block table.
-// q is [T, nh, d] with q_stride elements between tokens; out is [T, nh*d].
+// q is [T, nh, d] with q_stride elements between tokens; keys have d elements, values dv (K
+// pages [kv head, page_size, d], V pages [kv head, dv, page_size]); out is [T, nh*dv].
 int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                         const void* v_cache, const int32_t* table, int table_stride,
                         const int32_t* positions, const int32_t* token_req,
-                        const int32_t* slots, int T, int nh, int nkv, int d, int page_size,
+                        const int32_t* slots, int T, int nh, int nkv, int d, int dv, int page_size,
                         int num_pages, float scale, int window, int dtype, kvc_stream stream);
+
+// What kvc_rope_kv_write does, for heads whose keys (d) and values (dv) may differ in size,
+// with a norm of every q and k head before the rotation: rows of qkv are [nh q heads of d |
+// nkv k heads of d | nkv v heads of dv], row_stride elements apart.  With q_gain and k_gain
+// ([d] each, shared by all heads; both null: no norm) a head becomes gain * x / sqrt(mean(x^2)
+// + eps); then its first rot_dim elements are rotated by cos/sin [T, rot_dim / 2].  q and k are
+// rewritten in place; with write_kv, k goes to K[page, kv head, offset, :] and v to V[page, kv
+// head, :, offset] at kv_slot[t] (as kvc_kv_slots gives it).
+int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache, void* v_cache,
+                              const float* q_gain, const float* k_gain, float eps,
+                              const float* cos_tab, const float* sin_tab, int rot_dim,
+                              int interleaved, const int32_t* kv_slot, int T, int nh, int nkv, int d,
+                              int dv, int page_size, int write_kv, int dtype, kvc_stream stream);
+
+// residual += delta (skipped when delta is null); out = (residual - mean) / sqrt(var + eps) *
+// weight + bias (bias may be null), var the mean of the squared deviations; rounded to dt.
+int kvc_add_layernorm(void* out, float* residual, const void* delta, const float* weight,
+                      const float* bias, float eps, int T, int H, int dtype, kvc_stream stream);
+
+// out[t] = (1 / n) * sum_b gain_b * x_b[t] / sqrt(mean(x_b[t]^2) + eps) over n <= 4 branches of
+// float32 rows [T, H]; host_x and host_gain are host arrays of n device pointers.
+int kvc_rms_branches_mean(void* out, const float* const* host_x, const float* const* host_gain,
+                          int n, float eps, int T, int H, int dtype, kvc_stream stream);
+
+// out[t] = [a[t] | b[t]] ([T, 2H] of dt from two float32 [T, H]);  x[t, :] += v[:] (float32).
+int kvc_concat2(void* out, const float* a, const float* b, int T, int H, int dtype, kvc_stream stream);
+int kvc_add_row(float* x, const float* v, int T, int H, kvc_stream stream);
+
+// ---- mixers with a state of fixed size per request (recurrent.hip).  q_start [R+1], positions
+// [T], token_req [T] (-1: padding), slots [R] describe the flattened batch; a request whose
+// first token of the step is at position 0 starts from a zero state, any other from its slot's.
+//
+// Causal convolution per channel: out[t, c] = act(bias[c] + sum_j weight[c, K-1-j] * in(p - j)),
+// act 0 none or 1 silu, in() being zero before the sequence's start; state [slots, K-1, C]
+// float32 holds the K-1 inputs before the step and, with update_state, afterwards those before
+// the next.  x and out are rows of their dtypes with strides (x may be columns of a wider row).
+int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
+                    int x_dtype, const float* weight, const float* bias, float* state,
+                    const int32_t* positions, const int32_t* token_req, const int32_t* q_start,
+                    const int32_t* slots, int T, int R, int C, int K, int act, int update_state,
+                    kvc_stream stream);
+// Gates of the real-gated linear recurrent unit on u [T, W] float32, W in nb blocks: r =
+// sigmoid(wa[b] u_b + ba), i = sigmoid(wi[b] u_b + bi) (wa, wi [nb, W/nb, W/nb] float32, [out,
+// in]); a_out = exp(-c_decay * r * softplus(lam)); drive = sqrt(1 - a^2) * i * u.
+int kvc_rglru_gates(float* a_out, float* drive, const float* u, const float* wa, const float* wi,
+                    const float* ba, const float* bi, const float* lam, float c_decay, int T, int W,
+                    int nb, kvc_stream stream);
+// S_t = a_t S_(t-1) + drive_t per channel along each request (state [slots, W] float32);
+// out[t] = S_t * gelu_tanh(y[t]).
+int kvc_rglru_scan(void* out, int out_dtype, const float* a, const float* drive, const void* y,
+                   int64_t y_stride, int y_dtype, float* state, const int32_t* positions,
+                   const int32_t* token_req, const int32_t* q_start, const int32_t* slots, int R,
+                   int W, kvc_stream stream);
+// State-space recurrence with a scalar decay per head: xbc [T, >= nh*P + 2*G*N] float32 rows
+// hold x (nh heads of P), then B and C (G groups of N); per head h of group h / (nh / G):
+// dt = softplus(dt_raw[t, h] + dt_bias[h]); S = exp(-exp(a_log[h]) dt) S + dt B x^T (S [N, P],
+// state [slots, nh, N, P] float32); y[t, h] = S^T C + d_skip[h] x, y [T, nh*P] float32.
+// N at most kvc_ssm_scan_max_state().
+int kvc_ssm_scan_max_state(void);
+int kvc_ssm_scan(float* y, const float* xbc, int64_t xbc_stride, const void* dt_raw,
+                 int64_t dt_stride, int dt_dtype, const float* dt_bias, const float* a_log,
+                 const float* d_skip, float* state, const int32_t* positions,
+                 const int32_t* token_req, const int32_t* q_start, const int32_t* slots, int R,
+                 int nh, int P, int N, int G, kvc_stream stream);
+// out[t, c] = gain[c] * v / sqrt(mean of v^2 over c's part + eps), v = y[t, c] * silu(z[t, c]),
+// the width cut into `groups` equal parts.
+int kvc_gated_group_rmsnorm(void* out, int out_dtype, const float* y, const void* z,
+                            int64_t z_stride, int z_dtype, const float* gain, float eps, int T,
+                            int width, int groups, kvc_stream stream);
 
 // The same attention for bfloat16 steps of single tokens on the matrix cores, a block of
 // several waves per (token, kv head, split), which also does what kvc_rope_kv_write does for

@@ -19,7 +19,8 @@ class LayerCall:
 
     ``cache_index`` addresses the cache planes of this entry's group (None: the layer's
     mixer keeps no paged cache); ``write_cache`` is False when the entry reads the cache
-    another entry wrote.  ``state_index`` addresses the layer's fixed-size state array.
+    another entry wrote.  ``state_index`` addresses the layer's fixed-size state array, or the
+    first of them; ``state_indices`` all of them, in the order of the mixer's ``state_needs``.
     """
 
     exec_index: int
@@ -28,6 +29,7 @@ class LayerCall:
     cache_index: int | None = None
     write_cache: bool = True
     state_index: int | None = None
+    state_indices: tuple[int, ...] = ()
 
 
 @dataclass

@@ -14,7 +14,7 @@ import torch
 from kvcore_amd.engine.context import LayerCall, StepContext
 from kvcore_amd.ops import library as ops
 from kvcore_amd.parts import base as parts
-from kvcore_amd.parts.base import CacheNeed, ParamSpec, Part, Runtime, StateNeed
+from kvcore_amd.parts.base import CacheNeed, ParamSpec, Part, Runtime, StateNeed, checkpoint_name
 
 from .spec import ModelSpec
 
@@ -49,6 +49,7 @@ class BuiltParts:
     final_norm: parts.Norm
     blocks: list
     owned: list  # (checkpoint prefix, part), in the order parameters are declared
+    stream_ops: list = None
 
 
 def build_parts(spec: ModelSpec) -> BuiltParts:
@@ -72,10 +73,15 @@ def build_parts(spec: ModelSpec) -> BuiltParts:
     for i, pe in enumerate(positions):
         prefix = spec.position_prefixes[i] if spec.position_prefixes else f"model.positions.{i}"
         owned.append((prefix, pe))
+    stream_ops = [parts.STREAM_OPS.build(s) for s in spec.stream_ops]
+    if spec.stream_op_prefixes and len(spec.stream_op_prefixes) != len(stream_ops):
+        raise ValueError("stream_op_prefixes must name every stream op")
+    for i, op in enumerate(stream_ops):
+        owned.append((spec.stream_op_prefixes[i] if spec.stream_op_prefixes else f"model.stream_ops.{i}", op))
     for layer, block in zip(spec.layers, blocks):
         for sub, part in block.children().items():
             owned.append((f"{layer.prefix}.{sub}", part))
-    return BuiltParts(positions, embed, head, final_norm, blocks, owned)
+    return BuiltParts(positions, embed, head, final_norm, blocks, owned, stream_ops)
 
 
 class DecoderModel:
@@ -91,6 +97,7 @@ class DecoderModel:
         self.head = built.head
         self.final_norm = built.final_norm
         self.blocks = built.blocks
+        self.stream_ops = built.stream_ops
         self._owned = built.owned
         for _, part in self._owned:
             part.setup(self.runtime)
@@ -131,13 +138,16 @@ class DecoderModel:
                     g = group_of[need]
                     plane = planes[g]
                     planes[g] += 1
-            state_need = mixer.state_need()
-            state_index = None
-            if state_need is not None:
-                state_index = len(states)
+            state_indices = []
+            for state_need in mixer.state_needs():
+                state_indices.append(len(states))
                 states.append(StateArraySpec(state_need))
-            calls.append(LayerCall(e, entry.layer, g, plane, write, state_index))
+            if entry.before is not None and not 0 <= entry.before < len(self.stream_ops):
+                raise ValueError(f"schedule entry {e} names stream op {entry.before}, which does not exist")
+            calls.append(LayerCall(e, entry.layer, g, plane, write,
+                                   state_indices[0] if state_indices else None, tuple(state_indices)))
         self.calls = calls
+        self.schedule = schedule
         self.cache_groups = [CacheGroupSpec(n, c) for n, c in zip(needs, planes)]
         self.state_arrays = states
 
@@ -164,7 +174,7 @@ class DecoderModel:
         out: dict[str, tuple[BoundParam, int, int]] = {}
         for bp in self.params.values():
             for src in bp.spec.resolved_sources():
-                out[f"{bp.prefix}.{src.name}"] = (bp, src.row, src.rows)
+                out[checkpoint_name(bp.prefix, src.name)] = (bp, src.row, src.rows)
         return out
 
     def optional_checkpoint_names(self) -> set[str]:
@@ -252,9 +262,25 @@ class DecoderModel:
         for pe in self.positions:
             pe.prepare(ctx)
             pe.embed(residual, ctx)
+        embedded = None
+        if any(op.needs_embedded for op in self.stream_ops):
+            embedded = ctx.buf("embedded", H, torch.float32)
+            embedded.copy_(residual)
         delta = None
         for i, call in enumerate(self.calls):
-            nxt = self.blocks[self.calls[i + 1].layer_index] if i + 1 < len(self.calls) else None
+            entry = self.schedule[i]
+            if entry.before is not None:
+                if delta is not None:  # what the layer before left pending joins the stream first
+                    if isinstance(delta, (ops.ScaledRows, ops.NormedRows)):
+                        raise RuntimeError("a stream op follows a block that folded the next norm")
+                    ops.residual_add(residual, delta)
+                    delta = None
+                self.stream_ops[entry.before].forward(residual, embedded, ctx, entry.before_arg)
+            # a block may leave its last sum and the next block's first norm to the products
+            # around them only when nothing rewrites the stream in between
+            nxt = None
+            if i + 1 < len(self.calls) and self.schedule[i + 1].before is None:
+                nxt = self.blocks[self.calls[i + 1].layer_index]
             delta = self.blocks[call.layer_index].forward(delta, residual, ctx, call, next_block=nxt)
         hidden = ctx.buf("final_hidden", H)
         self.final_norm.forward_fused(hidden, residual, delta)

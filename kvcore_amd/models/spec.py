@@ -25,10 +25,14 @@ class LayerSpec:
 @dataclass(frozen=True)
 class ScheduleEntry:
     """Run ``layer``.  ``cache_from`` names an earlier schedule entry (by its index in the
-    schedule) whose cache this entry reads instead of writing its own."""
+    schedule) whose cache this entry reads instead of writing its own.  ``before`` names a
+    stream op (an index into ``ModelSpec.stream_ops``) that rewrites the residual stream right
+    before this entry's layer, with ``before_arg`` as its argument."""
 
     layer: int
     cache_from: int | None = None
+    before: int | None = None
+    before_arg: int = 0
 
 
 @dataclass(frozen=True)
@@ -40,6 +44,10 @@ class ModelSpec:
     final_norm: PartSpec
     positions: tuple[PartSpec, ...] = ()
     schedule: tuple[ScheduleEntry, ...] = ()
+    # changes of the whole stream that schedule entries name (``ScheduleEntry.before``), and
+    # their checkpoint prefixes (empty: "model.stream_ops.<i>")
+    stream_ops: tuple[PartSpec, ...] = ()
+    stream_op_prefixes: tuple[str, ...] = ()
     tie_word_embeddings: bool = False
     # the embedding and the head, chosen by kind like every other part; None stands for the
     # plain token embedding and the linear head (tied as ``tie_word_embeddings`` says) of

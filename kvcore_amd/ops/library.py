@@ -46,7 +46,17 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
-        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
+        "kvc_qk_norm_rope_kv_write": [P, L, P, P, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
+        "kvc_add_layernorm": [P, P, P, P, P, F, I, I, I, P],
+        "kvc_rms_branches_mean": [P, P, P, I, F, I, I, I, P],
+        "kvc_concat2": [P, P, P, I, I, I, P],
+        "kvc_add_row": [P, P, I, I, P],
+        "kvc_causal_conv": [P, L, I, P, L, I, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "kvc_rglru_gates": [P, P, P, P, P, P, P, P, F, I, I, I, P],
+        "kvc_rglru_scan": [P, I, P, P, P, L, I, P, P, P, P, P, I, I, P],
+        "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+        "kvc_gated_group_rmsnorm": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
                                  F, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
@@ -84,6 +94,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.kvc_last_variant.argtypes = [c_int]
     lib.kvc_argmax_static_capacity.restype = c_int
     lib.kvc_argmax_static_capacity.argtypes = []
+    lib.kvc_ssm_scan_max_state.restype = c_int
+    lib.kvc_ssm_scan_max_state.argtypes = []
 
 
 def load(build_if_missing: bool = True) -> ctypes.CDLL:
@@ -316,14 +328,16 @@ def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
                     slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-                    window: int = 0) -> None:
-    """``q`` is a ``[T, >= nh*d]`` view whose rows hold the query heads first."""
+                    window: int = 0, dv: int | None = None) -> None:
+    """``q`` is a ``[T, >= nh*d]`` view whose rows hold the query heads first.  ``dv``: the size
+    of a value head where it differs from a key head's ``d`` (``out`` is ``[T, nh*dv]``)."""
     T = out.shape[0]
-    if out.shape != (T, nh * d) or not out.is_contiguous():
-        raise KernelError("paged_attention: out must be contiguous [T, nh*d]")
+    dv = d if dv is None else dv
+    if out.shape != (T, nh * dv) or not out.is_contiguous():
+        raise KernelError("paged_attention: out must be contiguous [T, nh*dv]")
     if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
         raise KernelError("paged_attention: q does not fit")
-    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "paged_attention")
+    num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "paged_attention", dv)
     if k_cache.dtype != out.dtype:
         raise KernelError("paged_attention: cache dtype differs from the queries'")
     if positions.numel() < T or token_req.numel() < T:
@@ -332,8 +346,40 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(table, "table", torch.int32), table.shape[1],
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(slots, "slots", torch.int32), T, nh, nkv, d, page_size, num_pages, float(scale),
+        _dev(slots, "slots", torch.int32), T, nh, nkv, d, dv, page_size, num_pages, float(scale),
         int(window), _code(out, "out"), _stream()), "kvc_paged_attention")
+
+
+def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                          cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
+                          kv_slot: torch.Tensor, nh: int, nkv: int, d: int, dv: int,
+                          q_gain: torch.Tensor | None = None, k_gain: torch.Tensor | None = None,
+                          eps: float = 0.0, write_kv: bool = True) -> None:
+    """Rows of ``qkv`` are ``[nh heads of d | nkv heads of d | nkv heads of dv]``.  With gains
+    (float32 ``[d]``, shared by all heads) every q and k head is first divided by its root mean
+    square (``eps`` inside the root) and multiplied by the gain; then the first ``rot_dim``
+    elements are rotated; q and k are rewritten in place, k and v stored at ``kv_slot``
+    (``k_cache [pages, nkv, page_size, d]``, ``v_cache [pages, nkv, dv, page_size]``)."""
+    T = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < (nh + nkv) * d + nkv * dv:
+        raise KernelError(f"qk_norm_rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit the heads")
+    _check_cache(k_cache, v_cache, nkv, d, "qk_norm_rope_kv_write", dv)
+    page_size = k_cache.shape[2]
+    if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+        raise KernelError("qk_norm_rope_kv_write: cache dtype differs from qkv")
+    if rot_dim and (cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape):
+        raise KernelError("qk_norm_rope_kv_write: rotary tables do not fit")
+    if kv_slot.numel() < T:
+        raise KernelError("qk_norm_rope_kv_write: kv_slot too short")
+    for g in (q_gain, k_gain):
+        if g is not None and (g.shape != (d,) or g.dtype != torch.float32):
+            raise KernelError("qk_norm_rope_kv_write: a gain must be float32 [d]")
+    _check(load().kvc_qk_norm_rope_kv_write(
+        qkv.data_ptr(), qkv.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        None if q_gain is None else _dev(q_gain, "q_gain"), None if k_gain is None else _dev(k_gain, "k_gain"),
+        float(eps), _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), int(rot_dim),
+        int(bool(interleaved)), _dev(kv_slot, "kv_slot", torch.int32), T, nh, nkv, d, dv, page_size,
+        int(write_kv), _code(qkv, "qkv"), _stream()), "kvc_qk_norm_rope_kv_write")
 
 
 def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
@@ -513,14 +559,17 @@ def prefill_attention_rotates(rot_dim: int, interleaved: bool) -> bool:
     return rot_dim > 0 and rot_dim % (32 if interleaved else 64) == 0
 
 
-def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int, who: str) -> tuple[int, int]:
-    """K pages are ``[pages, nkv, page_size, d]``, V pages ``[pages, nkv, d, page_size]``."""
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, d: int, who: str,
+                 dv: int | None = None) -> tuple[int, int]:
+    """K pages are ``[pages, nkv, page_size, d]``, V pages ``[pages, nkv, dv, page_size]``
+    (``dv`` None: values as wide as keys)."""
+    dv = d if dv is None else dv
     if k_cache.dim() != 4 or v_cache.dim() != 4:
         raise KernelError(f"{who}: cache planes must be 4-D")
     num_pages, ckv, page_size, cd = k_cache.shape
-    if (ckv, cd) != (nkv, d) or tuple(v_cache.shape) != (num_pages, nkv, d, page_size):
+    if (ckv, cd) != (nkv, d) or tuple(v_cache.shape) != (num_pages, nkv, dv, page_size):
         raise KernelError(f"{who}: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
-                          f"{nkv} kv heads of {d}")
+                          f"{nkv} kv heads of {d} and {dv}")
     if k_cache.dtype != v_cache.dtype:
         raise KernelError(f"{who}: K and V planes differ in dtype")
     return num_pages, page_size
@@ -952,6 +1001,173 @@ def choose_product(M: int, N: int, K: int, *, few_rows_ok: bool = True, shared_r
     if shared_rows_ok and SKINNY_PREFERRED_ROWS < M <= MID_ROWS_WIDE and N >= 65536:
         return "shared rows"
     return "vendor"
+
+
+def add_layernorm(out: torch.Tensor, residual: torch.Tensor, delta: torch.Tensor | None,
+                  weight: torch.Tensor, bias: torch.Tensor | None, eps: float) -> None:
+    """``residual += delta`` (float32, in place); ``out = (residual - mean) / sqrt(var + eps) *
+    weight + bias`` with the variance as the mean of the squared deviations."""
+    T, H = residual.shape
+    if out.shape != (T, H) or weight.shape != (H,) or (delta is not None and delta.shape != (T, H)) \
+            or (bias is not None and bias.shape != (H,)):
+        raise KernelError("add_layernorm: shapes do not match")
+    if delta is not None and delta.dtype != out.dtype:
+        raise KernelError("add_layernorm: delta and out must share a dtype")
+    _check(load().kvc_add_layernorm(_dev(out, "out"), _dev(residual, "residual", torch.float32),
+                                    None if delta is None else _dev(delta, "delta"),
+                                    _dev(weight, "weight", torch.float32),
+                                    None if bias is None else _dev(bias, "bias", torch.float32),
+                                    float(eps), T, H, _code(out, "out"), _stream()), "kvc_add_layernorm")
+
+
+def rms_branches_mean(out: torch.Tensor, branches: list[tuple[torch.Tensor, torch.Tensor]], eps: float) -> None:
+    """``out = mean_b(gain_b * x_b / rms(x_b))`` over up to four ``(x_b [T, H] float32, gain_b [H]
+    float32)``, every branch divided by its own root mean square (``eps`` inside the root)."""
+    T, H = out.shape
+    n = len(branches)
+    if not 1 <= n <= 4 or not out.is_contiguous():
+        raise KernelError("rms_branches_mean: one to four branches, a contiguous result")
+    xs = (c_void_p * n)()
+    gs = (c_void_p * n)()
+    for b, (x, g) in enumerate(branches):
+        if x.shape != (T, H) or g.shape != (H,):
+            raise KernelError("rms_branches_mean: shapes do not match")
+        xs[b], gs[b] = _dev(x, "x", torch.float32), _dev(g, "gain", torch.float32)
+    _check(load().kvc_rms_branches_mean(_dev(out, "out"), xs, gs, n, float(eps), T, H, _code(out, "out"),
+                                        _stream()), "kvc_rms_branches_mean")
+
+
+def concat2(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
+    """``out [T, 2H] = [a | b]`` from float32 ``a, b [T, H]``, rounded to ``out``'s dtype."""
+    T, H = a.shape
+    if b.shape != (T, H) or out.shape != (T, 2 * H):
+        raise KernelError("concat2: shapes do not match")
+    _check(load().kvc_concat2(_dev(out, "out"), _dev(a, "a", torch.float32), _dev(b, "b", torch.float32),
+                              T, H, _code(out, "out"), _stream()), "kvc_concat2")
+
+
+def add_row(x: torch.Tensor, v: torch.Tensor) -> None:
+    """``x[t, :] += v`` on float32 rows."""
+    T, H = x.shape
+    if v.shape != (H,):
+        raise KernelError("add_row: shapes do not match")
+    _check(load().kvc_add_row(_dev(x, "x", torch.float32), _dev(v, "v", torch.float32), T, H, _stream()),
+           "kvc_add_row")
+
+
+def _rows(t: torch.Tensor, name: str, cols: int) -> tuple[int, int, int]:
+    """(pointer, row stride, dtype code) of rows that may be columns of a wider tensor."""
+    if t.dim() != 2 or t.stride(1) != 1 or t.shape[1] != cols or not t.is_cuda:
+        raise KernelError(f"{name}: expects GPU rows of {cols} contiguous elements, got {tuple(t.shape)}")
+    return t.data_ptr(), t.stride(0), _code(t, name)
+
+
+def causal_conv(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
+                state: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
+                q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int, act: str = "none",
+                update_state: bool = True) -> None:
+    """Causal convolution per channel over each request's tokens (see the C header): ``x [T, C]``
+    (a column view is fine), ``weight [C, K]`` float32 with the last column the current token's,
+    ``state [slots, K-1, C]`` float32 (read, and with ``update_state`` rewritten)."""
+    T, C = x.shape
+    K = weight.shape[1]
+    if weight.shape != (C, K) or (bias is not None and bias.shape != (C,)):
+        raise KernelError("causal_conv: weight or bias does not fit")
+    if state.dim() != 3 or tuple(state.shape[1:]) != (K - 1, C) or state.dtype != torch.float32:
+        raise KernelError("causal_conv: state must be float32 [slots, K-1, C]")
+    if out.shape[0] != T or positions.numel() < T or token_req.numel() < T or q_start.numel() < num_reqs + 1:
+        raise KernelError("causal_conv: index arrays or out too short")
+    o_ptr, o_stride, o_code = _rows(out, "out", C)
+    x_ptr, x_stride, x_code = _rows(x, "x", C)
+    _check(load().kvc_causal_conv(
+        o_ptr, o_stride, o_code, x_ptr, x_stride, x_code, _dev(weight, "weight", torch.float32),
+        None if bias is None else _dev(bias, "bias", torch.float32), _dev(state, "state"),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs, C, K,
+        {"none": 0, "silu": 1}[act], int(update_state), _stream()), "kvc_causal_conv")
+
+
+def rglru_gates(a_out: torch.Tensor, drive: torch.Tensor, u: torch.Tensor, wa: torch.Tensor,
+                wi: torch.Tensor, ba: torch.Tensor, bi: torch.Tensor, lam: torch.Tensor,
+                c_decay: float) -> None:
+    """Decay ``a = exp(-c_decay * sigmoid(wa u + ba) * softplus(lam))`` and driven input
+    ``sqrt(1 - a^2) * sigmoid(wi u + bi) * u`` of the gated linear recurrent unit, the gate
+    matrices block-diagonal ``[blocks, W/blocks, W/blocks]``; everything float32."""
+    T, W = u.shape
+    nb = wa.shape[0]
+    if W % nb or wa.shape != (nb, W // nb, W // nb) or wi.shape != wa.shape:
+        raise KernelError("rglru_gates: gate matrices do not fit")
+    if a_out.shape != (T, W) or drive.shape != (T, W) or ba.numel() != W or bi.numel() != W or lam.numel() != W:
+        raise KernelError("rglru_gates: shapes do not match")
+    f = torch.float32
+    _check(load().kvc_rglru_gates(_dev(a_out, "a_out", f), _dev(drive, "drive", f), _dev(u, "u", f),
+                                  _dev(wa, "wa", f), _dev(wi, "wi", f), _dev(ba, "ba", f), _dev(bi, "bi", f),
+                                  _dev(lam, "lam", f), float(c_decay), T, W, nb, _stream()), "kvc_rglru_gates")
+
+
+def rglru_scan(out: torch.Tensor, a: torch.Tensor, drive: torch.Tensor, y: torch.Tensor,
+               state: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
+               q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int) -> None:
+    """``S_t = a_t S_(t-1) + drive_t`` per channel along each request, ``out[t] = S_t *
+    gelu_tanh(y[t])``; ``state [slots, W]`` float32 is read (a request at position 0 starts
+    from zero) and rewritten."""
+    T, W = a.shape
+    if drive.shape != (T, W) or out.shape != (T, W) or not out.is_contiguous() or state.shape[1:] != (W,):
+        raise KernelError("rglru_scan: shapes do not match")
+    y_ptr, y_stride, y_code = _rows(y, "y", W)
+    _check(load().kvc_rglru_scan(
+        _dev(out, "out"), _code(out, "out"), _dev(a, "a", torch.float32), _dev(drive, "drive", torch.float32),
+        y_ptr, y_stride, y_code, _dev(state, "state", torch.float32),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, W, _stream()),
+        "kvc_rglru_scan")
+
+
+def ssm_scan_max_state() -> int:
+    return int(load().kvc_ssm_scan_max_state())
+
+
+def ssm_scan(y: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
+             a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, *, positions: torch.Tensor,
+             token_req: torch.Tensor, q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int,
+             heads: int, head_dim: int, state_size: int, groups: int) -> None:
+    """The state-space recurrence with a scalar decay per head (see the C header): ``xbc [T, heads
+    * head_dim + 2 * groups * state_size]`` float32 (x, B, C after their convolution), ``dt_raw
+    [T, heads]`` (a column view is fine), ``state [slots, heads, state_size, head_dim]`` float32,
+    ``y [T, heads * head_dim]`` float32."""
+    T = xbc.shape[0]
+    inner = heads * head_dim
+    if y.shape != (T, inner) or not y.is_contiguous() or y.dtype != torch.float32:
+        raise KernelError("ssm_scan: y must be contiguous float32 [T, heads * head_dim]")
+    if tuple(state.shape[1:]) != (heads, state_size, head_dim) or state.dtype != torch.float32:
+        raise KernelError("ssm_scan: state must be float32 [slots, heads, state_size, head_dim]")
+    if dt_bias.numel() != heads or a_log.numel() != heads or d_skip.numel() != heads:
+        raise KernelError("ssm_scan: a value per head for dt_bias, a_log and d_skip")
+    x_ptr, x_stride, x_code = _rows(xbc, "xbc", inner + 2 * groups * state_size)
+    if x_code != 0:
+        raise KernelError("ssm_scan: xbc must be float32")
+    d_ptr, d_stride, d_code = _rows(dt_raw, "dt_raw", heads)
+    f = torch.float32
+    _check(load().kvc_ssm_scan(
+        y.data_ptr(), x_ptr, x_stride, d_ptr, d_stride, d_code, _dev(dt_bias, "dt_bias", f),
+        _dev(a_log, "a_log", f), _dev(d_skip, "d_skip", f), _dev(state, "state"),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, heads,
+        head_dim, state_size, groups, _stream()), "kvc_ssm_scan")
+
+
+def gated_group_rmsnorm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, gain: torch.Tensor,
+                        eps: float, groups: int) -> None:
+    """``out = gain * v / rms_part(v)`` with ``v = y * silu(z)``: the gate first, then the norm
+    in ``groups`` equal parts of the width.  ``y`` float32, ``z`` a column view of any dtype."""
+    T, width = y.shape
+    if out.shape != (T, width) or not out.is_contiguous() or not y.is_contiguous() or gain.shape != (width,):
+        raise KernelError("gated_group_rmsnorm: shapes do not match")
+    z_ptr, z_stride, z_code = _rows(z, "z", width)
+    _check(load().kvc_gated_group_rmsnorm(
+        _dev(out, "out"), _code(out, "out"), _dev(y, "y", torch.float32), z_ptr, z_stride, z_code,
+        _dev(gain, "gain", torch.float32), float(eps), T, width, groups, _stream()),
+        "kvc_gated_group_rmsnorm")
 
 
 def table_update(table: torch.Tensor, triples: torch.Tensor, n: int) -> None:

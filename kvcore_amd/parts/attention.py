@@ -100,48 +100,80 @@ class PagedAttention(Mixer):
 
     @property
     def takes_sink(self) -> bool:  # the output product's rows are whole heads
-        return self.q_size % 8 == 0
+        return self.o_size % 8 == 0 and not self.float32_result
 
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, bias: bool = False, window: int = 0, page_size: int | None = None,
+                 v_head_dim: int | None = None, qk_norm_eps: float | None = None,
+                 tensor_names: dict[str, str] | None = None, float32_result: bool = False,
                  position: PositionEncoding | None = None) -> None:
+        """``v_head_dim``: the size of a value head where it differs from ``head_dim``, the
+        size of a query and key head.  ``qk_norm_eps`` (None: no such norm): every query and
+        key head is divided by its root mean square, eps inside the root, and multiplied by a
+        gain of ``head_dim`` values shared by all heads, before the rotation.  ``tensor_names``
+        renames checkpoint tensors (keys ``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``;
+        values relative to the part's prefix).  ``float32_result``: the output rows are
+        float32 sums, for a consumer that normalises them."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
-        if head_dim % 16 or head_dim > 256:
+        v_head_dim = head_dim if v_head_dim is None else v_head_dim
+        plain = v_head_dim == head_dim and qk_norm_eps is None
+        if plain and (head_dim % 16 or head_dim > 256):
             raise ValueError(f"head size {head_dim} is not supported (multiples of 16 up to 256)")
+        if not 0 < head_dim <= 256 or not 0 < v_head_dim <= 256:
+            raise ValueError(f"head sizes {head_dim} and {v_head_dim} are not supported (1 to 256)")
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
+        self.v_head_dim = v_head_dim
+        self.qk_norm_eps = qk_norm_eps
         self.scale = scale
         self.bias = bias
         self.window = window
         self.page_size = page_size  # None: the engine's block size
         self.position = position
+        self.float32_result = float32_result
         self.q_size = num_heads * head_dim
         self.kv_size = num_kv_heads * head_dim
+        self.v_size = num_kv_heads * v_head_dim
+        self.o_size = num_heads * v_head_dim
+        self.plain = plain
+        self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight",
+                      "o": "o_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
+                      "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+                      "o_bias": "o_proj.bias", **(tensor_names or {})}
 
     def param_specs(self) -> list[ParamSpec]:
-        total = self.q_size + 2 * self.kv_size
+        total = self.q_size + self.kv_size + self.v_size
+        n = self.names
 
-        def stacked(suffix: str) -> tuple[ParamSource, ...]:
+        def stacked(q: str, k: str, v: str) -> tuple[ParamSource, ...]:
             return (
-                ParamSource(f"q_proj.{suffix}", 0, self.q_size),
-                ParamSource(f"k_proj.{suffix}", self.q_size, self.kv_size),
-                ParamSource(f"v_proj.{suffix}", self.q_size + self.kv_size, self.kv_size),
+                ParamSource(n[q], 0, self.q_size),
+                ParamSource(n[k], self.q_size, self.kv_size),
+                ParamSource(n[v], self.q_size + self.kv_size, self.v_size),
             )
 
         specs = [
-            ParamSpec("qkv_proj.weight", (total, self.hidden_size), sources=stacked("weight")),
-            ParamSpec("o_proj.weight", (self.hidden_size, self.q_size)),
+            ParamSpec("qkv_proj.weight", (total, self.hidden_size), sources=stacked("q", "k", "v")),
+            ParamSpec("o_proj.weight", (self.hidden_size, self.o_size),
+                      sources=(ParamSource(n["o"], 0, self.hidden_size),)),
         ]
         if self.bias:
-            specs.append(ParamSpec("qkv_proj.bias", (total,), init="zeros", sources=stacked("bias")))
-            specs.append(ParamSpec("o_proj.bias", (self.hidden_size,), init="zeros"))
+            specs.append(ParamSpec("qkv_proj.bias", (total,), init="zeros",
+                                   sources=stacked("q_bias", "k_bias", "v_bias")))
+            specs.append(ParamSpec("o_proj.bias", (self.hidden_size,), init="zeros",
+                                   sources=(ParamSource(n["o_bias"], 0, self.hidden_size),)))
+        if self.qk_norm_eps is not None:
+            for key in ("q_norm", "k_norm"):
+                specs.append(ParamSpec(key, (self.head_dim,), kind="vector", init="gain",
+                                       sources=(ParamSource(n[key], 0, self.head_dim),)))
         return specs
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window, self.page_size)
+        return CacheNeed(((self.num_kv_heads, self.head_dim), (self.num_kv_heads, self.v_head_dim)),
+                         self.window, self.page_size)
 
     def check_limits(self, limits) -> None:
         """The decode kernel keeps the page ids of a split's key range in LDS; a block table
@@ -153,7 +185,7 @@ class PagedAttention(Mixer):
             raise ValueError(
                 f"{type(self).__name__} keeps its cache in {need.dtype} beside a model in "
                 f"{self.runtime.dtype}: the attention kernels read keys and values in the model's dtype")
-        if self.runtime.dtype != torch.bfloat16 or not ops.decode_attention_supported(
+        if not self._same_sizes() or self.runtime.dtype != torch.bfloat16 or not ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, limits.page_size, self.runtime.dtype):
             return
         widest = ops.decode_attention_max_table(self.num_heads, self.num_kv_heads, self.head_dim)
@@ -167,27 +199,47 @@ class PagedAttention(Mixer):
     def product_weights(self) -> tuple[str, ...]:
         return ("qkv_proj.weight", "o_proj.weight")
 
+    def _same_sizes(self) -> bool:
+        """Keys and values of one size: what the matrix-core kernels serve."""
+        return self.v_head_dim == self.head_dim
+
     def forward(self, x, ctx, call, sink=None):
         p = self.params
-        qkv = ctx.buf("attn_qkv", self.q_size + 2 * self.kv_size)
+        # step buffers are named by their width: layers of one model may differ in size
+        qkv = ctx.buf(_sized("attn_qkv", self.q_size + self.kv_size + self.v_size, self.plain),
+                      self.q_size + self.kv_size + self.v_size)
         ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
 
         group = ctx.groups[call.group_index]
-        # K pages [kv_heads, page, d]; V pages [kv_heads, d, page]: the keys of a page lie
+        # K pages [kv_heads, page, d]; V pages [kv_heads, dv, page]: the keys of a page lie
         # side by side, which is how the matrix cores want the values
         k_cache = group.plane(call.cache_index, 0, self.num_kv_heads, group.page_size, self.head_dim)
-        v_cache = group.plane(call.cache_index, 1, self.num_kv_heads, self.head_dim, group.page_size)
+        v_cache = group.plane(call.cache_index, 1, self.num_kv_heads, self.v_head_dim, group.page_size)
         rot = self.position.rotary(ctx) if self.position is not None else None
         if rot is None:
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
             rot_dim, interleaved = 0, False
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
-        attn = ctx.buf("attn_out", self.q_size)
+        attn = ctx.buf(_sized("attn_out", self.o_size, self.plain), self.o_size)
         common = dict(table=group.table, positions=ctx.positions, token_req=ctx.token_req,
                       slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
                       scale=self.scale, window=self.window)
-        if ctx.max_query_len == 1 and ops.decode_attention_supported(
+        # with a norm of the heads, or values of another size than the keys, one kernel norms,
+        # rotates and writes the cache; the attention kernels then take q and the cache as they are
+        prepared = not self.plain
+        if prepared:
+            kv_slot = self._kv_slots(ctx, call, group, k_cache)
+            ops.qk_norm_rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
+                                      interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
+                                      nkv=self.num_kv_heads, d=self.head_dim, dv=self.v_head_dim,
+                                      q_gain=p.get("q_norm"), k_gain=p.get("k_norm"),
+                                      eps=self.qk_norm_eps or 0.0, write_kv=call.write_cache)
+            rot_dim, interleaved = 0, False
+            cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
+        if not self._same_sizes():
+            ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_head_dim, **common)
+        elif ctx.max_query_len == 1 and ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
             # single tokens: rotation, cache write and attention in one kernel on the matrix
             # cores, a block per (token, kv head, split)
@@ -200,33 +252,26 @@ class PagedAttention(Mixer):
                 # for the largest at once, since a buffer that grows drops the graphs
                 most = (decode_target_blocks() // self.num_kv_heads + 1 + max(T, ctx.buffers.seq_capacity)) \
                     * self.num_heads
-                part_o = ctx.buffers.get("attn_part_o", T * self.num_heads * nsplit, self.head_dim,
+                part_o = ctx.buffers.get(_sized("attn_part_o", self.head_dim, self.plain),
+                                         T * self.num_heads * nsplit, self.head_dim,
                                          torch.float32, reserve=most)
                 part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32,
                                           reserve=most)
             ops.decode_attention(attn, qkv, k_cache, v_cache, nsplit=nsplit, part_o=part_o,
                                  part_ml=part_ml, cos=cos, sin=sin, rot_dim=rot_dim,
-                                 interleaved=interleaved, write_kv=call.write_cache,
+                                 interleaved=interleaved, write_kv=call.write_cache and not prepared,
                                  token_rows=ctx.token_rows, **common)
         else:
-            # where each token's key and value go: once per step and cache group
-            slot_key = ("kv_slot", call.group_index)
-            kv_slot = ctx.scratch.get(slot_key)
-            if kv_slot is None:
-                kv_slot = ctx.buf(f"kv_slot_{call.group_index}", 1, torch.int32).view(-1)
-                ops.kv_slots(kv_slot, positions=ctx.positions, token_req=ctx.token_req,
-                             slots=ctx.slots, table=group.table, page_size=group.page_size,
-                             num_pages=k_cache.shape[0])
-                ctx.scratch[slot_key] = kv_slot
             on_matrix_cores = ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype)
             # the kernel for portions rotates the queries on their way in where it can, which
             # saves writing them and reading them again
             rotates = on_matrix_cores and ops.prefill_attention_rotates(rot_dim, interleaved)
-            ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
-                              interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
-                              nkv=self.num_kv_heads, d=self.head_dim, write_kv=call.write_cache,
-                              rotate_q=not rotates)
+            if not prepared:
+                ops.rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
+                                  interleaved=interleaved, kv_slot=self._kv_slots(ctx, call, group, k_cache),
+                                  nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
+                                  write_kv=call.write_cache, rotate_q=not rotates)
             if on_matrix_cores:
                 # portions of prompts (single tokens may ride along): tiles of query rows per
                 # block, and several blocks per tile where few rows meet many keys
@@ -237,7 +282,8 @@ class PagedAttention(Mixer):
                 if nsplit > 1:
                     # asked for at their largest at once: a buffer that grows drops the graphs
                     most = prefill_split_rows(self.num_kv_heads, self.num_heads // self.num_kv_heads) * self.num_heads
-                    part_o = ctx.buffers.get("attn_prefill_part_o", T * self.num_heads * nsplit,
+                    part_o = ctx.buffers.get(_sized("attn_prefill_part_o", self.head_dim, self.plain),
+                                             T * self.num_heads * nsplit,
                                              self.head_dim, torch.float32, reserve=most)
                     part_ml = ctx.buffers.get("attn_prefill_part_ml", T * self.num_heads * nsplit, 2,
                                               torch.float32, reserve=most)
@@ -252,9 +298,32 @@ class PagedAttention(Mixer):
                 ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
         if sink is not None:
             return ops.linear(sink, attn, p["o_proj.weight"], p.get("o_proj.bias"))
-        out = ctx.buf("mixer_out", self.hidden_size)
+        if self.float32_result:
+            out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
+        else:
+            out = ctx.buf("mixer_out", self.hidden_size)
         ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         return out
+
+    @staticmethod
+    def _kv_slots(ctx, call, group, k_cache):
+        """Where each token's key and value go: once per step and cache group."""
+        slot_key = ("kv_slot", call.group_index)
+        kv_slot = ctx.scratch.get(slot_key)
+        if kv_slot is None:
+            kv_slot = ctx.buf(f"kv_slot_{call.group_index}", 1, torch.int32).view(-1)
+            ops.kv_slots(kv_slot, positions=ctx.positions, token_req=ctx.token_req,
+                         slots=ctx.slots, table=group.table, page_size=group.page_size,
+                         num_pages=k_cache.shape[0])
+            ctx.scratch[slot_key] = kv_slot
+        return kv_slot
+
+
+def _sized(name: str, cols: int, plain: bool) -> str:
+    """The name of a step buffer: the plain attention of a model whose layers are all alike
+    keeps one buffer per role; the others name theirs by width, since a buffer whose width
+    changes from layer to layer would be allocated anew at every layer."""
+    return name if plain else f"{name}:{cols}"
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -33,6 +33,12 @@ class ParamSource:
     rows: int
 
 
+def checkpoint_name(prefix: str, name: str) -> str:
+    """The checkpoint tensor that a source names: ``prefix.name``, or the prefix itself for an
+    empty name (a part whose one tensor is called as the part is)."""
+    return f"{prefix}.{name}" if name else prefix
+
+
 @dataclass(frozen=True)
 class ParamSpec:
     """A parameter a part owns.
@@ -240,7 +246,27 @@ class Mixer(Part):
     def state_need(self) -> StateNeed | None:
         return None
 
+    def state_needs(self) -> tuple[StateNeed, ...]:
+        """Every array of per-request state that the mixer keeps (``state_need`` for a mixer
+        with one); ``LayerCall.state_indices`` names them in this order."""
+        need = self.state_need()
+        return () if need is None else (need,)
+
     def forward(self, x: torch.Tensor, ctx: "StepContext", call: "LayerCall") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class StreamOp(Part):
+    """A change of the whole residual stream between layers, named by a schedule entry
+    (``ScheduleEntry.before``): ``forward`` rewrites the float32 ``residual [T, H]`` in place
+    (what the layer before left pending has been added by then).  ``embedded`` is the
+    embedding's output for the step's tokens, kept for the ops that say ``needs_embedded``;
+    ``arg`` is the schedule entry's own number for the op (a pass count, say)."""
+
+    needs_embedded = False
+
+    def forward(self, residual: torch.Tensor, embedded: torch.Tensor | None, ctx: "StepContext",
+                arg: int) -> None:
         raise NotImplementedError
 
 
@@ -357,6 +383,7 @@ POSITION_ENCODINGS = _Registry("position encoding")
 BLOCKS = _Registry("block")
 EMBEDDINGS = _Registry("embedding")
 HEADS = _Registry("head")
+STREAM_OPS = _Registry("stream op")
 
 
 def register_mixer(kind: str, factory: Callable[..., Mixer], **kw: Any) -> None:
@@ -385,3 +412,7 @@ def register_embedding(kind: str, factory: Callable[..., Embedding], **kw: Any) 
 
 def register_head(kind: str, factory: Callable[..., Head], **kw: Any) -> None:
     HEADS.register(kind, factory, **kw)
+
+
+def register_stream_op(kind: str, factory: Callable[..., StreamOp], **kw: Any) -> None:
+    STREAM_OPS.register(kind, factory, **kw)

@@ -17,7 +17,8 @@ from .base import Block, FeedForward, Mixer, Norm, Part, register_block
 
 class PreNormBlock(Block):
     """``r += delta; a = mixer(norm_in(r)); r += a; out = ffn(norm_post(r))``, the last
-    sum left pending for the next block's first norm."""
+    sum left pending for the next block's first norm.  With a feed-forward of kind ``none`` the
+    block is ``r += delta; out = mixer(norm_in(r))``."""
 
     def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm],
                  mixer_name: str = "self_attn", ffn_name: str = "mlp",
@@ -27,11 +28,16 @@ class PreNormBlock(Block):
         left out, they are the first and the second norm that the layer lists."""
         super().__init__(mixer=mixer, ffn=ffn, norms=norms)
         listed = list(norms)
+        self.mixer_only = bool(getattr(ffn, "absent", False))
         if input_norm is None and listed:
             input_norm = listed[0]
         if post_norm is None:
             post_norm = next((n for n in listed if n != input_norm), None)
-        missing = [n for n in (input_norm, post_norm) if n not in norms]
+        if self.mixer_only:
+            post_norm = None
+            if input_norm not in norms:
+                raise ValueError(f"a pre-norm block needs a norm before the mixer; given {listed}")
+        missing = [n for n in (input_norm, post_norm) if n not in norms and not self.mixer_only]
         if missing or input_norm == post_norm:
             raise ValueError(f"a pre-norm block needs two norms, one before the mixer and one before the "
                              f"feed-forward; asked for {(input_norm, post_norm)}, given {listed}")
@@ -40,6 +46,8 @@ class PreNormBlock(Block):
         self.ffn_name = ffn_name
 
     def children(self) -> dict[str, Part]:
+        if self.mixer_only:
+            return {self.norm_names[0]: self.norms[self.norm_names[0]], self.mixer_name: self.mixer}
         return {
             self.norm_names[0]: self.norms[self.norm_names[0]],
             self.mixer_name: self.mixer,
@@ -70,6 +78,8 @@ class PreNormBlock(Block):
             x = ctx.buf("block_x", residual.shape[1])
             self.norms[self.norm_names[0]].forward_fused(x, residual, delta)
 
+        if self.mixer_only:  # x + mixer(norm(x)) and nothing more; the sum stays pending
+            return self.mixer.forward(x, ctx, call)
         post = self.norms[self.norm_names[1]]
         gain = None
         if self.mixer.takes_sink and ((fold and self.ffn.takes_scaled_rows) or sums):

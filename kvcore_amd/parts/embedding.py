@@ -13,20 +13,25 @@ import torch
 
 from kvcore_amd.ops import library as ops
 
-from .base import Embedding, Head, ParamSpec, register_embedding, register_head
+from .base import Embedding, Head, ParamSource, ParamSpec, register_embedding, register_head
 
 
 class TokenEmbedding(Embedding):
     """``scale`` multiplies the embedded rows (1.0 for Llama; some architectures use
     ``sqrt(hidden_size)``)."""
 
-    def __init__(self, *, vocab_size: int, hidden_size: int, scale: float = 1.0) -> None:
+    def __init__(self, *, vocab_size: int, hidden_size: int, scale: float = 1.0,
+                 weight_name: str = "weight") -> None:
+        """``weight_name``: the checkpoint tensor relative to the part's prefix (empty: the
+        prefix itself)."""
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.scale = float(scale)
+        self.weight_name = weight_name
 
     def param_specs(self) -> list[ParamSpec]:
-        return [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
+        return [ParamSpec("weight", (self.vocab_size, self.hidden_size),
+                          sources=(ParamSource(self.weight_name, 0, self.vocab_size),))]
 
     def forward(self, residual: torch.Tensor, token_ids: torch.Tensor) -> None:
         ops.embed(residual, self.params["weight"], token_ids, self.scale)
@@ -38,7 +43,7 @@ class LinearHead(Head):
     the embedding matrix to them."""
 
     def __init__(self, *, vocab_size: int, hidden_size: int, tied: bool = False, bias: bool = False,
-                 logit_scale: float = 1.0, soft_cap: float = 0.0) -> None:
+                 logit_scale: float = 1.0, soft_cap: float = 0.0, weight_name: str = "weight") -> None:
         if soft_cap < 0:
             raise ValueError(f"soft_cap must be positive when set, got {soft_cap}")
         self.vocab_size = vocab_size
@@ -47,9 +52,11 @@ class LinearHead(Head):
         self.bias = bias
         self.logit_scale = float(logit_scale)
         self.soft_cap = float(soft_cap)
+        self.weight_name = weight_name
 
     def param_specs(self) -> list[ParamSpec]:
-        specs = [] if self.tied else [ParamSpec("weight", (self.vocab_size, self.hidden_size))]
+        specs = [] if self.tied else [ParamSpec("weight", (self.vocab_size, self.hidden_size),
+                                                sources=(ParamSource(self.weight_name, 0, self.vocab_size),))]
         if self.bias:
             specs.append(ParamSpec("bias", (self.vocab_size,), init="zeros"))
         return specs

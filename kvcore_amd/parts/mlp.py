@@ -22,35 +22,51 @@ class SwiGLU(FeedForward):
     def takes_sink(self) -> bool:
         return self.intermediate_size % 8 == 0
 
-    def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False) -> None:
+    def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False,
+                 gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj",
+                 suffix: str = ".weight", sized_buffers: bool = False) -> None:
+        """``gate_name``, ``up_name`` and ``down_name`` are the checkpoint's names of the three
+        matrices relative to the part's prefix, ``suffix`` what follows each (biases end in
+        ``.bias``).  ``sized_buffers``: name the step buffers by their width, for a model whose
+        layers may differ in width (a buffer whose width changed from layer to layer would be
+        allocated anew at every layer)."""
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.bias = bias
+        self.names = (gate_name, up_name, down_name)
+        self.suffix = suffix
+        self.sized_buffers = sized_buffers
 
     def param_specs(self) -> list[ParamSpec]:
         I, H = self.intermediate_size, self.hidden_size
 
+        gate, up, down = self.names
+
         def stacked(suffix: str) -> tuple[ParamSource, ...]:
-            return (ParamSource(f"gate_proj.{suffix}", 0, I), ParamSource(f"up_proj.{suffix}", I, I))
+            return (ParamSource(gate + suffix, 0, I), ParamSource(up + suffix, I, I))
 
         specs = [
-            ParamSpec("gate_up_proj.weight", (2 * I, H), sources=stacked("weight")),
-            ParamSpec("down_proj.weight", (H, I)),
+            ParamSpec("gate_up_proj.weight", (2 * I, H), sources=stacked(self.suffix)),
+            ParamSpec("down_proj.weight", (H, I), sources=(ParamSource(down + self.suffix, 0, H),)),
         ]
         if self.bias:
-            specs.append(ParamSpec("gate_up_proj.bias", (2 * I,), init="zeros", sources=stacked("bias")))
-            specs.append(ParamSpec("down_proj.bias", (H,), init="zeros"))
+            specs.append(ParamSpec("gate_up_proj.bias", (2 * I,), init="zeros", sources=stacked(".bias")))
+            specs.append(ParamSpec("down_proj.bias", (H,), init="zeros",
+                                   sources=(ParamSource(down + ".bias", 0, H),)))
         return specs
 
     def product_weights(self) -> tuple[str, ...]:
         return ("gate_up_proj.weight", "down_proj.weight")
 
+    def _buf(self, name: str) -> str:
+        return f"{name}:{self.intermediate_size}" if self.sized_buffers else name
+
     def forward(self, x, ctx, call, sink=None):
         p = self.params
-        act = ctx.buf("ffn_act", self.intermediate_size)
+        act = ctx.buf(self._buf("ffn_act"), self.intermediate_size)
         # few rows: the product and the activation are one kernel and gate_up is never stored
         ops.linear_silu_mul(act, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"),
-                            lambda: ctx.buf("ffn_gate_up", 2 * self.intermediate_size))
+                            lambda: ctx.buf(self._buf("ffn_gate_up"), 2 * self.intermediate_size))
         if sink is not None:
             return ops.linear(sink, act, p["down_proj.weight"], p.get("down_proj.bias"))
         out = ctx.buf("ffn_out", self.hidden_size)
@@ -58,4 +74,14 @@ class SwiGLU(FeedForward):
         return out
 
 
+class NoFeedForward(FeedForward):
+    """A layer that has a mixer only: the block skips the second norm and the second sum."""
+
+    absent = True
+
+    def forward(self, x, ctx, call, sink=None):
+        raise RuntimeError("a layer without a feed-forward has nothing to run here")
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("none", NoFeedForward)

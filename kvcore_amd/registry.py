@@ -1,6 +1,6 @@
 """One registry from an architecture's name to how its model is made.
 
-The key is ``architectures[0]`` of config.json, with ``model_type`` as a second chance
+The key is ``architectures[0]`` of config.json (or its ``architecture``), with ``model_type`` as a second chance
 (the reference keys on ``model_type`` alone: kvcore/model/model_loader/
 default_loader.py:32-36,64-70).  An entry holds a parser from the raw config mapping to
 a typed configuration and a function from that configuration to a ``ModelSpec``.
@@ -40,6 +40,8 @@ def unregister_architecture(name: str) -> None:
 
 def resolve_architecture(config: Mapping[str, Any]) -> Architecture:
     names = list(config.get("architectures") or [])
+    if config.get("architecture"):  # some configurations name one architecture, in the singular
+        names.append(config["architecture"])
     if config.get("model_type"):
         names.append(config["model_type"])
     for name in names:
@@ -55,6 +57,11 @@ def _register_builtin() -> None:
     from kvcore_amd.models.llama import llama_spec
 
     register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec, aliases=("llama",))
+
+    from kvcore_amd.config.dirulorn_config import DirulornConfig
+    from kvcore_amd.models.dirulorn import dirulorn_spec
+
+    register_architecture("Dirulorn", DirulornConfig.from_dict, dirulorn_spec)
 
 
 _register_builtin()

@@ -164,12 +164,13 @@ def checkpoint_layout(model_spec) -> dict[str, tuple[tuple[int, ...], str, str]]
     """The checkpoint tensors a model of this spec reads: name -> (shape, init rule,
     kind), derived from the parts' declarations without allocating the model."""
     from kvcore_amd.models.decoder import build_parts
+    from kvcore_amd.parts.base import checkpoint_name
 
     layout: dict[str, tuple[tuple[int, ...], str, str]] = {}
     for prefix, part in build_parts(model_spec).owned:
         for ps in part.param_specs():
             for src in ps.resolved_sources():
-                layout[f"{prefix}.{src.name}"] = ((src.rows, *ps.shape[1:]), ps.init, ps.kind)
+                layout[checkpoint_name(prefix, src.name)] = ((src.rows, *ps.shape[1:]), ps.init, ps.kind)
     return layout
 
 
