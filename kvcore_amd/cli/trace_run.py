@@ -31,7 +31,7 @@ def parse_args(argv=None) -> argparse.Namespace:
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (each rounded up to 64)")
     p.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
-    p.add_argument("--max-num-seqs", type=int, default=8, help="request slots")
+    p.add_argument("--max-num-seqs", type=int, default=4, help="request slots (no more requests are live at a time)")
     p.add_argument("--device", default="cuda:0")
     p.add_argument("--poison-cache", action="store_true",
                    help="fill the cache with NaN first, so a read of a slot nobody wrote shows")
