@@ -222,8 +222,14 @@ class ModelRunner:
 
     # -------------------------------------------------------------------- bookkeeping
     def forget(self, slot: int) -> None:
-        """A request left its slot.  The next owner's pages are synced from scratch."""
+        """A request left its slot.  The next owner's pages are synced from scratch.  With
+        ``poison_pages`` the slot's rows of every state array become NaN (on the stream, behind
+        the steps launched so far), so that a next owner that read them would show."""
         self._slot_owner[slot] = None
+        if self.poison_pages:
+            for state in self.states:
+                if state.dtype.is_floating_point:
+                    state[slot].fill_(float("nan"))
 
     def poison(self, pages: Sequence[Sequence[int]]) -> None:
         """Fill the listed pages (one list per cache group) with NaN on the stream, behind the
@@ -239,11 +245,14 @@ class ModelRunner:
                     ops.fill_pages(plane, dev, len(ids), float("nan"), page_axis=1)
 
     def fill_cache(self, value: float) -> None:
-        """Overwrite every cache plane (tests fill with NaN so that a read outside a
-        request's own slots shows in the logits)."""
+        """Overwrite every cache plane and state array (tests fill with NaN so that a read
+        outside a request's own slots shows in the logits)."""
         for g in self.groups:
             for plane in g.storage:
                 plane.fill_(value)
+        for state in self.states:
+            if state.dtype.is_floating_point:
+                state.fill_(value)
 
     def cache_bytes(self) -> int:
         return sum(p.numel() * p.element_size() for g in self.groups for p in g.storage)

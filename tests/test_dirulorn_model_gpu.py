@@ -1,0 +1,202 @@
+"""The Dirulorn decoder in the engine against the plain implementation, under every way of
+cutting the work: whole prompts, prompts then single tokens, portions down to two tokens,
+unequal requests side by side, pages and state slots that are given back and used again, long
+decoding, and greedy generation through the engine's own entry point and scheduler."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from tests.dirulorn_helpers import CONFIGS, make_model_dir
+from tests.helpers import random_tokens
+from tests.plain import dirulorn as plain
+from tests.test_cuts_gpu import collect
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, (config, page) in CONFIGS.items():
+        folder = make_model_dir(tmp_path_factory.mktemp(f"dirulorn_{name}"), config, seed=31 + len(out))
+        cfg, weights = plain.load_model_folder(folder)
+        out[name] = (folder, cfg, weights, page)
+    return out
+
+
+_oracle: dict = {}
+
+
+def oracle(name, cfg, weights, tokens):
+    key = (name, tuple(tokens))
+    if key not in _oracle:
+        _oracle[key] = plain.forward(cfg, weights, tokens)
+    return _oracle[key]
+
+
+def session_for(folder, dtype, page, max_tokens, **kw):
+    from kvcore_amd.engine.replay import TraceSession
+
+    return TraceSession(str(folder), dtype, max_tokens=max_tokens, block_size=page, poison_cache=True, **kw)
+
+
+def compare(got, expect_by_id, dtype):
+    """Logit rows against the plain model's: the difference with its mean taken off, root mean
+    square over the vocabulary, relative to the root mean square of the row itself.  float32
+    differs by the order of its sums only; bfloat16 rounds activations to 8 bits at a dozen
+    places a layer."""
+    limit = 2e-4 if dtype == torch.float32 else 6e-2
+    assert got, "nothing was compared"
+    worst = 0.0
+    for (rid, pos), row in sorted(got.items()):
+        ref = expect_by_id[rid][pos]
+        assert torch.isfinite(row).all(), f"non-finite logits at {rid}:{pos}"
+        d = row - ref
+        d = d - d.mean()
+        err = float(d.pow(2).mean().sqrt() / (ref - ref.mean()).pow(2).mean().sqrt())
+        worst = max(worst, err)
+        assert err <= limit, f"{rid}:{pos} differs by {err:.3e} of its size (limit {limit})"
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompts_then_single_tokens_then_portions(models, name, dtype):
+    folder, cfg, weights, page = models[name]
+    V = cfg["vocab"]
+    tokens = random_tokens(75, V, 5)
+    want = {"a": oracle(name, cfg, weights, tokens)}
+    s = session_for(folder, dtype, page, 256)
+    # whole
+    got = collect(s, [{"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": list(range(75))}], "end": ["a"]}])
+    compare(got, want, dtype)
+    # a prompt, then token by token (the slot and the pages of the first run are used again)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": tokens[:40], "want": [0, 39]}], "end": []}]
+    for i in range(40, 75):
+        steps.append({"step": i, "entries": [{"id": "a", "tokens": tokens[i: i + 1], "want": [0]}],
+                      "end": ["a"] if i == 74 else []})
+    compare(collect(s, steps), want, dtype)
+    # portions of every size down to two tokens and one, cut inside pages
+    steps, at = [], 0
+    for n in (2, 3, 2, 1, 9, 2, 17, 1, 1, 2, 30, 5):
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": tokens[at: at + n],
+                                                       "want": list(range(n))}],
+                      "end": ["a"] if at + n == 75 else []})
+        at += n
+    assert at == 75
+    compare(collect(s, steps), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_unequal_requests_side_by_side_with_slots_used_again(models, name, dtype):
+    """Up to three live requests in two slots' worth of pages more than one needs: portions of
+    some beside single tokens of others, requests that pause, end and are followed by new ones
+    in the same slots and pages."""
+    folder, cfg, weights, page = models[name]
+    V = cfg["vocab"]
+    seqs = {"a": random_tokens(61, V, 1), "b": random_tokens(33, V, 2), "c": random_tokens(9, V, 3),
+            "d": random_tokens(47, V, 4), "e": random_tokens(2, V, 5), "f": random_tokens(1, V, 6)}
+    want = {k: oracle(name, cfg, weights, v) for k, v in seqs.items()}
+    s = session_for(folder, dtype, page, 192, max_num_seqs=3)
+    at = {k: 0 for k in seqs}
+
+    def entry(k, n, want_all=True):
+        lo = at[k]
+        n = min(n, len(seqs[k]) - lo)
+        at[k] += n
+        return {"id": k, "tokens": seqs[k][lo: lo + n], "want": list(range(n)) if want_all else [n - 1]}
+
+    plan = [
+        [("a", 20), ("b", 2)], [("a", 1), ("b", 13), ("c", 9)], [("a", 7), ("b", 1)],
+        [("b", 1), ("d", 2), ("a", 1)], [("d", 30), ("a", 1), ("b", 1)], [("a", 31)],
+        [("b", 15), ("d", 1)], [("d", 14), ("e", 2)], [("f", 1)],
+    ]
+    steps = []
+    for i, group in enumerate(plan):
+        entries = [entry(k, n) for k, n in group]
+        ended = [k for k, _ in group if at[k] == len(seqs[k])]
+        steps.append({"step": i, "entries": entries, "end": ended})
+    assert all(at[k] == len(v) for k, v in seqs.items())
+    compare(collect(s, steps), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+def test_long_decoding_through_graphs(models, dtype):
+    """Three hundred single tokens after a short prompt, two requests side by side (the steps of
+    single tokens are captured into a graph and replayed), one of them starting later."""
+    folder, cfg, weights, page = models["Q"]
+    V = cfg["vocab"]
+    seqs = {"a": random_tokens(330, V, 7), "b": random_tokens(290, V, 8)}
+    want = {k: oracle("Q", cfg, weights, v) for k, v in seqs.items()}
+    s = session_for(folder, dtype, page, 704)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": seqs["a"][:30], "want": [29]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": seqs["a"][30:31], "want": [0]},
+                                     {"id": "b", "tokens": seqs["b"][:10], "want": [9]}], "end": []}]
+    for i in range(280):
+        steps.append({"step": 2 + i, "entries": [{"id": "a", "tokens": seqs["a"][31 + i: 32 + i], "want": [0]},
+                                                 {"id": "b", "tokens": seqs["b"][10 + i: 11 + i], "want": [0]}],
+                      "end": []})
+    got = collect(s, steps)
+    assert s.runner.graph_replays > 200
+    compare(got, want, dtype)
+
+
+def test_attention_runs_on_the_matrix_cores_where_keys_and_values_are_alike(models):
+    """Keys and values of one size that the matrix-core kernels serve: in bfloat16 the norm and
+    rotation kernel prepares q and the cache, and those kernels do the attention."""
+    from kvcore_amd.ops import library as ops
+
+    folder, cfg, weights, page = models["Q"]
+    left = cfg["layers"][1]["mixer"]["left"]
+    assert ops.prefill_attention_supported(left["heads"], left["kv_heads"], left["dim"], page, torch.bfloat16)
+    assert ops.decode_attention_supported(left["heads"], left["kv_heads"], left["dim"], page, torch.bfloat16)
+    s = session_for(folder, torch.bfloat16, page, 128)
+    tokens = random_tokens(70, cfg["vocab"], 9)
+    s.run_step({"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": [69]}], "end": ["a"]})
+    assert ops.last_variant("prefill_attention").startswith("prefill_attention_kernel")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_greedy_generation_through_the_engine(models, name, dtype):
+    """``LLMEngine.generate`` with the scheduler cutting prompts into portions of 16 tokens:
+    every generated token is the plain model's greedy choice given the tokens before it (a
+    choice is skipped where the plain model's two best logits lie closer than rounding
+    can tell apart)."""
+    from kvcore_amd import CacheConfig, KVCoreConfig, ModelConfig, SamplingParams, SchedulerConfig
+    from kvcore_amd.engine.llm_engine import GenerationRequest, LLMEngine
+
+    folder, cfg, weights, page = models[name]
+    V = cfg["vocab"]
+    config = KVCoreConfig(
+        model_config=ModelConfig(model=str(folder), dtype="float32" if dtype == torch.float32 else "bfloat16",
+                                 max_model_len=128),
+        cache_config=CacheConfig(block_size=page, num_gpu_blocks=40),
+        scheduler_config=SchedulerConfig(max_num_seqs=3, max_num_scheduled_tokens=24,
+                                         long_prefill_token_threshold=16))
+    engine = LLMEngine(config)
+    prompts = {"r0": random_tokens(37, V, 11), "r1": random_tokens(5, V, 12), "r2": random_tokens(50, V, 13),
+               "r3": random_tokens(18, V, 14), "r4": random_tokens(1, V, 15)}
+    params = SamplingParams(max_tokens=12, temperature=0.0)
+    outs = engine.generate([GenerationRequest(k, params, prompt_token_ids=tuple(v)) for k, v in prompts.items()])
+    by_id = {o.request_id: list(o.output_token_ids) for o in outs}
+    assert set(by_id) == set(prompts)
+    margin = 1e-4 if dtype == torch.float32 else 5e-2
+    checked = 0
+    for rid, prompt in prompts.items():
+        gen = by_id[rid]
+        assert len(gen) == 12
+        logits = plain.forward(cfg, weights, prompt + gen)
+        for i, tok in enumerate(gen):
+            row = logits[len(prompt) + i - 1]
+            top = torch.topk(row, 2).values
+            if float(top[0] - top[1]) < margin * float(row.std()):
+                continue
+            assert int(torch.argmax(row)) == tok, f"{rid}: token {i}"
+            checked += 1
+    assert checked > 40
