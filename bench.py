@@ -20,7 +20,10 @@ Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 r
 with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
 first token of one N-token prompt in portions of 2,048), ``--sweep`` (decode at further
 batch sizes and context lengths, a line each with its share of the memory bandwidth);
-``--model 1b|70b`` and ``--batch`` change the shape.
+``--model 1b|70b`` and ``--batch`` change the shape.  ``--dirulorn s|m`` times the Dirulorn
+decoder (state-space layers beside attention-with-recurrence layers) at layer sizes of a real
+model, prefill and decode, next to a Llama of the same width, depth, feed-forward and head
+counts, a line each.
 """
 
 from __future__ import annotations
@@ -60,6 +63,109 @@ HBM_PEAK = 8.0e12          # bytes/s, MI355X
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
+def _dirulorn_layers(n, width, heads, kv, ff, lru_width, lru_blocks, ssm_heads, ssm_groups):
+    ssm = {"type": "mamba2", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"heads": ssm_heads, "vdim": 64, "state": 128, "groups": ssm_groups, "conv": 4,
+                     "norm_groups": ssm_groups}}
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"left": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 0.125,
+                              "rot": {"dims": 32, "base": 500000.0,
+                                      "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+                     "right": {"width": lru_width, "blocks": lru_blocks, "conv": 4}}}
+    return [ssm if i % 2 == 0 else par for i in range(n)]
+
+
+# Dirulorn at the layer sizes of a real model: every other layer a state-space mixer (an inner
+# width of twice the model's, states of 128 rows a head), the rest attention (keys of 64, values
+# of 128) beside a gated linear recurrent block; and the Llama each is set against
+DIRULORN_SHAPES = {
+    "s": ({"architecture": "Dirulorn", "vocab": 32000, "width": 1024, "norm": {"eps": 1e-5},
+           "layers": _dirulorn_layers(8, 1024, 16, 4, 4096, 1280, 8, 32, 4)},
+          dict(LLAMA32_1B, num_hidden_layers=8, hidden_size=1024, num_attention_heads=16,
+               num_key_value_heads=4, head_dim=64, intermediate_size=4096, vocab_size=32000,
+               tie_word_embeddings=False)),
+    "m": ({"architecture": "Dirulorn", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5},
+           "layers": _dirulorn_layers(16, 2048, 32, 8, 8192, 2560, 10, 64, 8)},
+          dict(LLAMA32_1B, num_hidden_layers=16, vocab_size=32000, tie_word_embeddings=False)),
+}
+
+
+def bench_dirulorn(args) -> int:
+    """Prefill (one 2,048-token prompt in one step) and decode (batch 8 and 64 from 512-token
+    prompts) of a Dirulorn shape and of the Llama of equal size, through the whole engine; a
+    JSON line per model and workload."""
+    import torch
+
+    from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig,
+                            SamplingParams, SchedulerConfig)
+    from kvcore_amd.engine.engine_core import EngineCore
+    from kvcore_amd.engine.runner import build_model
+
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    shapes = DIRULORN_SHAPES[args.dirulorn]
+    which = {"both": (0, 1), "dirulorn": (0,), "llama": (1,)}[args.dirulorn_only]
+    for index in which:
+        cfg = shapes[index]
+        name = f"dirulorn-{args.dirulorn}" if index == 0 else f"llama-of-dirulorn-{args.dirulorn}"
+        vocab = cfg["vocab"] if index == 0 else cfg["vocab_size"]
+        model = build_model(".", dtype, device, load_format="random", seed=0, config_override=cfg)
+        seqs = 64
+        pages = seqs * -(-(PREFILL_TOKENS + 512 + 256) // args.page_size) + 1
+        engine = EngineCore(KVCoreConfig(
+            model_config=ModelConfig(model=".", dtype=args.dtype, max_model_len=8192),
+            load_config=LoadConfig(load_format="random", seed=0),
+            cache_config=CacheConfig(block_size=args.page_size, num_gpu_blocks=pages),
+            scheduler_config=SchedulerConfig(max_num_seqs=seqs, max_num_scheduled_tokens=PREFILL_TOKENS,
+                                             max_num_partial_prefills=seqs, max_long_partial_prefills=seqs),
+            device_config=DeviceConfig(device=device)), model=model)
+        rng = random.Random(0)
+        counter = [0]
+
+        def new_request(n_prompt, n_new):
+            counter[0] += 1
+            engine.add_request(f"{name}-{counter[0]}", SamplingParams(max_tokens=n_new, ignore_eos=True, temperature=0.0),
+                               prompt_token_ids=[rng.randrange(vocab) for _ in range(n_prompt)])
+
+        times = []
+        for _ in range(4):
+            new_request(PREFILL_TOKENS, 1)
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t_start)
+            while engine.has_unfinished_requests():
+                engine.step()
+        sec = sorted(times[1:])[1]
+        params = model.num_param_bytes()
+        print(json.dumps({"model": name, "workload": "prefill", "dtype": args.dtype, "tokens": PREFILL_TOKENS,
+                          "ms": round(sec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
+                          "param_gib": round(params / 2**30, 3)}), flush=True)
+        for batch in (8, 64):
+            steps, warmup = args.steps, min(args.warmup, 8)
+            for _ in range(batch):
+                new_request(512, warmup + steps + 8 + batch * 512 // PREFILL_TOKENS)
+            while any(r.num_computed_tokens < r.num_prompt_tokens for r in engine.scheduler.requests.values()):
+                engine.step()
+            for _ in range(warmup):
+                engine.step()
+            torch.cuda.synchronize()
+            t_start = time.perf_counter()
+            for _ in range(steps):
+                engine.step()
+            torch.cuda.synchronize()
+            sec = (time.perf_counter() - t_start) / steps
+            engine.abort_requests(None)
+            print(json.dumps({"model": name, "workload": "decode", "dtype": args.dtype, "batch": batch,
+                              "ms_per_step": round(sec * 1e3, 4), "tokens_per_s": round(batch / sec, 1),
+                              "weights_gb_per_s": round(params / sec / 1e9, 1)}), flush=True)
+        del engine, model
+        torch.cuda.empty_cache()
+    return 0
+
+
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -93,6 +199,11 @@ def parse_args():
                    help="check the tokens before timing: against the plain implementation on the CPU "
                         "(default for the 8b and 1b shapes), finite logits and tokens in range only, "
                         "or not at all")
+    p.add_argument("--dirulorn", default=None, choices=sorted(DIRULORN_SHAPES),
+                   help="instead of the default run: prefill and decode of the Dirulorn decoder at this "
+                        "size, and of a Llama of the same width, depth and feed-forward; a line each")
+    p.add_argument("--dirulorn-only", default="both", choices=["both", "dirulorn", "llama"],
+                   help="with --dirulorn: run one of the two models only (for profiling)")
     p.add_argument("--sweep", action="store_true",
                    help="instead of the default run: decode at batch 1..64 and at contexts of 8k, 32k "
                         "and 128k tokens, a line each")
@@ -243,6 +354,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.dirulorn:
+        return bench_dirulorn(args)
     import torch
 
     from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig,
