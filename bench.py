@@ -129,7 +129,7 @@ def bench_dirulorn(args) -> int:
                                prompt_token_ids=[rng.randrange(vocab) for _ in range(n_prompt)])
 
         times = []
-        for _ in range(4):
+        for _ in range(4 if args.dirulorn_workload in ("all", "prefill") else 0):
             new_request(PREFILL_TOKENS, 1)
             torch.cuda.synchronize()
             t_start = time.perf_counter()
@@ -138,12 +138,15 @@ def bench_dirulorn(args) -> int:
             times.append(time.perf_counter() - t_start)
             while engine.has_unfinished_requests():
                 engine.step()
-        sec = sorted(times[1:])[1]
         params = model.num_param_bytes()
-        print(json.dumps({"model": name, "workload": "prefill", "dtype": args.dtype, "tokens": PREFILL_TOKENS,
-                          "ms": round(sec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
-                          "param_gib": round(params / 2**30, 3)}), flush=True)
+        if times:
+            sec = sorted(times[1:])[1]
+            print(json.dumps({"model": name, "workload": "prefill", "dtype": args.dtype, "tokens": PREFILL_TOKENS,
+                              "ms": round(sec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
+                              "param_gib": round(params / 2**30, 3)}), flush=True)
         for batch in (8, 64):
+            if args.dirulorn_workload not in ("all", f"decode{batch}"):
+                continue
             steps, warmup = args.steps, min(args.warmup, 8)
             for _ in range(batch):
                 new_request(512, warmup + steps + 8 + batch * 512 // PREFILL_TOKENS)
@@ -204,6 +207,8 @@ def parse_args():
                         "size, and of a Llama of the same width, depth and feed-forward; a line each")
     p.add_argument("--dirulorn-only", default="both", choices=["both", "dirulorn", "llama"],
                    help="with --dirulorn: run one of the two models only (for profiling)")
+    p.add_argument("--dirulorn-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
+                   help="with --dirulorn: run one of the workloads only (for profiling)")
     p.add_argument("--sweep", action="store_true",
                    help="instead of the default run: decode at batch 1..64 and at contexts of 8k, 32k "
                         "and 128k tokens, a line each")

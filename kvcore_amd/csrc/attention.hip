@@ -186,9 +186,15 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
 // offset, :]; the value heads of dv elements are copied to V[page, kv head, :, offset].
 namespace {
 
+constexpr int kMaxValuePlanes = 4;
+template <typename T>
+struct ValuePlanes {
+  T* plane[kMaxValuePlanes];
+};
+
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
-    T* __restrict__ qkv, int64_t row_stride, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    T* __restrict__ qkv, int64_t row_stride, T* __restrict__ k_cache, ValuePlanes<T> v_planes, int v_chunk,
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
     int interleaved, const int32_t* __restrict__ kv_slot, int nh, int nkv, int d, int dv,
@@ -260,15 +266,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     __syncthreads();
   }
   if (!store_kv) return;
+  // element i of a value head goes to plane i / v_chunk, V[page, kv head, i % v_chunk, offset]
   const T* vrow = row + static_cast<int64_t>(nh + nkv) * d;
-  const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * dv + off;
-  for (int w = threadIdx.x; w < nkv * dv; w += blockDim.x)
-    v_cache[v_base + static_cast<int64_t>(w) * page_size] = vrow[w];  // w = head * dv + i
+  const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * v_chunk + off;
+  for (int w = threadIdx.x; w < nkv * dv; w += blockDim.x) {
+    const int head = w / dv, i = w - head * dv;
+    const int c = i / v_chunk, ii = i - c * v_chunk;
+    v_planes.plane[c][v_base + (static_cast<int64_t>(head) * v_chunk + ii) * page_size] = vrow[w];
+  }
 }
 
 }  // namespace
 
-extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache, void* v_cache,
+extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache,
+                                         void* const* host_v_planes, int num_v_planes,
                                          const float* q_gain, const float* k_gain, float eps,
                                          const float* cos_tab, const float* sin_tab, int rot_dim,
                                          int interleaved, const int32_t* kv_slot, int T, int nh,
@@ -283,12 +294,16 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
     return kvc_fail("kvc_qk_norm_rope_kv_write: rows too short for the heads");
   if ((q_gain == nullptr) != (k_gain == nullptr))
     return kvc_fail("kvc_qk_norm_rope_kv_write: gains for both q and k, or for neither");
+  if (num_v_planes < 1 || num_v_planes > kMaxValuePlanes || dv % num_v_planes)
+    return kvc_fail("kvc_qk_norm_rope_kv_write: one to four value planes that divide the value size");
   if (T == 0) return 0;
+  const int v_chunk = dv / num_v_planes;
   KVC_DISPATCH_DTYPE(
-      dtype, Tp,
+      dtype, Tp, ValuePlanes<Tp> planes{};
+      for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
       hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<Tp>, dim3(T), dim3(256), 0,
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
-                         static_cast<Tp*>(k_cache), static_cast<Tp*>(v_cache), q_gain, k_gain, eps,
+                         static_cast<Tp*>(k_cache), planes, v_chunk, q_gain, k_gain, eps,
                          cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,
                          write_kv));
   return kvc_check_launch("kvc_qk_norm_rope_kv_write");

@@ -126,9 +126,12 @@ int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* 
 // ([d] each, shared by all heads; both null: no norm) a head becomes gain * x / sqrt(mean(x^2)
 // + eps); then its first rot_dim elements are rotated by cos/sin [T, rot_dim / 2].  q and k are
 // rewritten in place; with write_kv, k goes to K[page, kv head, offset, :] and v to V[page, kv
-// head, :, offset] at kv_slot[t] (as kvc_kv_slots gives it).
-int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache, void* v_cache,
-                              const float* q_gain, const float* k_gain, float eps,
+// head, :, offset] at kv_slot[t] (as kvc_kv_slots gives it).  The values may be kept in
+// num_v_planes (1 to 4) planes of dv / num_v_planes elements a head each (host_v_planes: a host
+// array of their device pointers): element i of a value head then lies in plane i / (dv /
+// num_v_planes), so that kernels whose keys and values are of one size can serve a plane each.
+int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_cache,
+                              void* const* host_v_planes, int num_v_planes, const float* q_gain, const float* k_gain, float eps,
                               const float* cos_tab, const float* sin_tab, int rot_dim,
                               int interleaved, const int32_t* kv_slot, int T, int nh, int nkv, int d,
                               int dv, int page_size, int write_kv, int dtype, kvc_stream stream);

@@ -47,7 +47,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
-        "kvc_qk_norm_rope_kv_write": [P, L, P, P, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
+        "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_add_layernorm": [P, P, P, P, P, F, I, I, I, P],
         "kvc_rms_branches_mean": [P, P, P, I, F, I, I, I, P],
         "kvc_concat2": [P, P, P, I, I, I, P],
@@ -350,7 +350,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         int(window), _code(out, "out"), _stream()), "kvc_paged_attention")
 
 
-def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor,
+                          v_cache: "torch.Tensor | list[torch.Tensor]",
                           cos: torch.Tensor, sin: torch.Tensor, *, rot_dim: int, interleaved: bool,
                           kv_slot: torch.Tensor, nh: int, nkv: int, d: int, dv: int,
                           q_gain: torch.Tensor | None = None, k_gain: torch.Tensor | None = None,
@@ -359,13 +360,21 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     (float32 ``[d]``, shared by all heads) every q and k head is first divided by its root mean
     square (``eps`` inside the root) and multiplied by the gain; then the first ``rot_dim``
     elements are rotated; q and k are rewritten in place, k and v stored at ``kv_slot``
-    (``k_cache [pages, nkv, page_size, d]``, ``v_cache [pages, nkv, dv, page_size]``)."""
+    (``k_cache [pages, nkv, page_size, d]``, ``v_cache [pages, nkv, dv, page_size]``, or a list of
+    up to four planes ``[pages, nkv, dv / n, page_size]`` that each hold a slice of every value
+    head)."""
     T = qkv.shape[0]
     if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < (nh + nkv) * d + nkv * dv:
         raise KernelError(f"qk_norm_rope_kv_write: qkv shape {tuple(qkv.shape)} does not fit the heads")
-    _check_cache(k_cache, v_cache, nkv, d, "qk_norm_rope_kv_write", dv)
+    planes = list(v_cache) if isinstance(v_cache, (list, tuple)) else [v_cache]
+    if not 1 <= len(planes) <= 4 or dv % len(planes):
+        raise KernelError("qk_norm_rope_kv_write: one to four value planes that divide the value size")
+    for plane in planes:
+        _check_cache(k_cache, plane, nkv, d, "qk_norm_rope_kv_write", dv // len(planes))
+        if plane.dtype != qkv.dtype:
+            raise KernelError("qk_norm_rope_kv_write: cache dtype differs from qkv")
     page_size = k_cache.shape[2]
-    if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+    if k_cache.dtype != qkv.dtype:
         raise KernelError("qk_norm_rope_kv_write: cache dtype differs from qkv")
     if rot_dim and (cos.shape[0] < T or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape):
         raise KernelError("qk_norm_rope_kv_write: rotary tables do not fit")
@@ -374,8 +383,9 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     for g in (q_gain, k_gain):
         if g is not None and (g.shape != (d,) or g.dtype != torch.float32):
             raise KernelError("qk_norm_rope_kv_write: a gain must be float32 [d]")
+    pointers = (c_void_p * len(planes))(*[_dev(plane, "v_cache") for plane in planes])
     _check(load().kvc_qk_norm_rope_kv_write(
-        qkv.data_ptr(), qkv.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        qkv.data_ptr(), qkv.stride(0), _dev(k_cache, "k_cache"), pointers, len(planes),
         None if q_gain is None else _dev(q_gain, "q_gain"), None if k_gain is None else _dev(k_gain, "k_gain"),
         float(eps), _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32), int(rot_dim),
         int(bool(interleaved)), _dev(kv_slot, "kv_slot", torch.int32), T, nh, nkv, d, dv, page_size,

@@ -139,6 +139,11 @@ class PagedAttention(Mixer):
         self.v_size = num_kv_heads * v_head_dim
         self.o_size = num_heads * v_head_dim
         self.plain = plain
+        # values wider than the keys by a whole factor (up to four) are kept in that many cache
+        # planes of the keys' size, so that the kernels for keys and values of one size serve them
+        factor = v_head_dim // head_dim if v_head_dim % head_dim == 0 else 0
+        self.v_planes = factor if 1 < factor <= 4 else 1
+        self.v_plane_dim = v_head_dim // self.v_planes
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight",
                       "o": "o_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
                       "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
@@ -172,8 +177,8 @@ class PagedAttention(Mixer):
         return specs
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(((self.num_kv_heads, self.head_dim), (self.num_kv_heads, self.v_head_dim)),
-                         self.window, self.page_size)
+        values = ((self.num_kv_heads, self.v_plane_dim),) * self.v_planes
+        return CacheNeed(((self.num_kv_heads, self.head_dim), *values), self.window, self.page_size)
 
     def check_limits(self, limits) -> None:
         """The decode kernel keeps the page ids of a split's key range in LDS; a block table
@@ -200,8 +205,8 @@ class PagedAttention(Mixer):
         return ("qkv_proj.weight", "o_proj.weight")
 
     def _same_sizes(self) -> bool:
-        """Keys and values of one size: what the matrix-core kernels serve."""
-        return self.v_head_dim == self.head_dim
+        """Keys and values of one size in every plane: what the matrix-core kernels serve."""
+        return self.v_plane_dim == self.head_dim
 
     def forward(self, x, ctx, call, sink=None):
         p = self.params
@@ -212,9 +217,11 @@ class PagedAttention(Mixer):
 
         group = ctx.groups[call.group_index]
         # K pages [kv_heads, page, d]; V pages [kv_heads, dv, page]: the keys of a page lie
-        # side by side, which is how the matrix cores want the values
+        # side by side, which is how the matrix cores want the values.  Values wider than the
+        # keys by a whole factor lie in that many planes of the keys' size
         k_cache = group.plane(call.cache_index, 0, self.num_kv_heads, group.page_size, self.head_dim)
-        v_cache = group.plane(call.cache_index, 1, self.num_kv_heads, self.v_head_dim, group.page_size)
+        v_planes = [group.plane(call.cache_index, 1 + c, self.num_kv_heads, self.v_plane_dim, group.page_size)
+                    for c in range(self.v_planes)]
         rot = self.position.rotary(ctx) if self.position is not None else None
         if rot is None:
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
@@ -222,25 +229,52 @@ class PagedAttention(Mixer):
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
         attn = ctx.buf(_sized("attn_out", self.o_size, self.plain), self.o_size)
-        common = dict(table=group.table, positions=ctx.positions, token_req=ctx.token_req,
-                      slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
-                      scale=self.scale, window=self.window)
         # with a norm of the heads, or values of another size than the keys, one kernel norms,
         # rotates and writes the cache; the attention kernels then take q and the cache as they are
         prepared = not self.plain
         if prepared:
             kv_slot = self._kv_slots(ctx, call, group, k_cache)
-            ops.qk_norm_rope_kv_write(qkv, k_cache, v_cache, cos, sin, rot_dim=rot_dim,
+            ops.qk_norm_rope_kv_write(qkv, k_cache, v_planes, cos, sin, rot_dim=rot_dim,
                                       interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
                                       nkv=self.num_kv_heads, d=self.head_dim, dv=self.v_head_dim,
                                       q_gain=p.get("q_norm"), k_gain=p.get("k_norm"),
                                       eps=self.qk_norm_eps or 0.0, write_kv=call.write_cache)
             rot_dim, interleaved = 0, False
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
+        if self.v_planes == 1:
+            self._attend(attn, qkv, k_cache, v_planes[0], ctx, call, group, cos, sin, rot_dim, interleaved, prepared)
+        else:
+            # the same scores against each plane of the values; the planes' results, each [T, heads
+            # * plane size], are then laid side by side within every head
+            T, m, part = ctx.num_tokens, self.v_planes, self.num_heads * self.v_plane_dim
+            parts = ctx.buffers.get(f"attn_planes:{part}", m * T, part, ctx.dtype,
+                                    reserve=m * ctx.buffers.token_capacity)
+            for c in range(m):
+                self._attend(parts[c * T: (c + 1) * T], qkv, k_cache, v_planes[c], ctx, call, group, cos, sin,
+                             rot_dim, interleaved, prepared)
+            attn.view(T, self.num_heads, m, self.v_plane_dim).copy_(
+                parts.view(m, T, self.num_heads, self.v_plane_dim).permute(1, 2, 0, 3))
+        if sink is not None:
+            return ops.linear(sink, attn, p["o_proj.weight"], p.get("o_proj.bias"))
+        if self.float32_result:
+            out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
+        else:
+            out = ctx.buf("mixer_out", self.hidden_size)
+        ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
+        return out
+
+    def _attend(self, attn, qkv, k_cache, v_cache, ctx, call, group, cos, sin, rot_dim, interleaved, prepared):
+        """The attention itself into ``attn [T, heads * plane size]`` over one plane of values,
+        by the kernel that serves the step's shape.  ``prepared``: q is ready and the cache is
+        written; otherwise the kernels chosen here rotate and write on their way."""
+        common = dict(table=group.table, positions=ctx.positions, token_req=ctx.token_req,
+                      slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
+                      scale=self.scale, window=self.window)
+        x_dtype = qkv.dtype
         if not self._same_sizes():
-            ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_head_dim, **common)
+            ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_plane_dim, **common)
         elif ctx.max_query_len == 1 and ops.decode_attention_supported(
-                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype):
+                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x_dtype):
             # single tokens: rotation, cache write and attention in one kernel on the matrix
             # cores, a block per (token, kv head, split)
             T = ctx.num_tokens
@@ -263,7 +297,7 @@ class PagedAttention(Mixer):
                                  token_rows=ctx.token_rows, **common)
         else:
             on_matrix_cores = ctx.max_query_len > 1 and self.scale > 0 and ops.prefill_attention_supported(
-                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x.dtype)
+                self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x_dtype)
             # the kernel for portions rotates the queries on their way in where it can, which
             # saves writing them and reading them again
             rotates = on_matrix_cores and ops.prefill_attention_rotates(rot_dim, interleaved)
@@ -296,14 +330,6 @@ class PagedAttention(Mixer):
                                          if rotates else {}))
             else:
                 ops.paged_attention(attn, qkv, k_cache, v_cache, **common)
-        if sink is not None:
-            return ops.linear(sink, attn, p["o_proj.weight"], p.get("o_proj.bias"))
-        if self.float32_result:
-            out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
-        else:
-            out = ctx.buf("mixer_out", self.hidden_size)
-        ops.linear(out, attn, p["o_proj.weight"], p.get("o_proj.bias"))
-        return out
 
     @staticmethod
     def _kv_slots(ctx, call, group, k_cache):

@@ -43,8 +43,9 @@ CONFIG_P = {
     "loop": {"start": 1, "stop": 3, "times": 3},
 }
 
-# keys and values of one size (64) with four query heads a kv head: in bfloat16 with pages of
-# 16 the matrix-core attention kernels serve it; no loop
+# keys and values of one size (64) with four query heads a kv head, and values of three times
+# the keys' size (kept as three planes of 64): in bfloat16 with pages of 16 the matrix-core
+# attention kernels serve both; no loop
 CONFIG_Q = {
     "architecture": "Dirulorn", "vocab": 320, "width": 128, "norm": {"eps": 1e-6},
     "layers": [
@@ -53,7 +54,7 @@ CONFIG_Q = {
          "mixer": _par(8, 2, 64, 64, 0.125, {"dims": 32, "base": 10000.0, "scaling":
                        {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 64}}, 128, 2, 4)},
         {"type": "parallel", "mlp": {"kind": "dense", "ff": 256},
-         "mixer": _par(4, 4, 64, 64, 0.11, None, 96, 1, 2)},
+         "mixer": _par(4, 2, 64, 192, 0.11, None, 96, 1, 2)},  # values three times as wide as keys
     ],
 }
 
@@ -65,7 +66,7 @@ CONFIG_R = {
     "layers": [
         {"type": "mamba2", "mlp": {"kind": "dense", "ff": 40}, "mixer": _ssm(1, 5, 3, 1, 1, 1)},
         {"type": "parallel", "mlp": None,
-         "mixer": _par(1, 1, 16, 16, 1.0, {"dims": 2, "base": 2.0}, 40, 1, 1)},
+         "mixer": _par(1, 1, 16, 32, 1.0, {"dims": 2, "base": 2.0}, 40, 1, 1)},
         {"type": "mamba2", "mlp": None, "mixer": _ssm(7, 1, 9, 7, 2, 7)},
     ],
     "loop": {"start": 0, "stop": 3, "times": 2},

@@ -265,19 +265,20 @@ def test_state_space_recurrence_whole_and_in_steps(ops, nh, P, N, G):
 
 
 # -------------------------------------------------------------------------- attention
-def attention_setup(ops, T_cap, nkv, d, dv, page, dtype):
+def attention_setup(ops, T_cap, nkv, d, dv, page, dtype, planes=1):
     pages = -(-T_cap // page) + 3
     kc = torch.full((pages, nkv, page, d), float("nan"), dtype=dtype, device=DEV)
-    vc = torch.full((pages, nkv, dv, page), float("nan"), dtype=dtype, device=DEV)
-    return kc, vc
+    vc = [torch.full((pages, nkv, dv // planes, page), float("nan"), dtype=dtype, device=DEV)
+          for _ in range(planes)]
+    return kc, vc[0] if planes == 1 else vc
 
 
 def run_attention_in_steps(ops, qkv, cuts, nh, nkv, d, dv, scale, freqs, interleaved, gains, eps, page, dtype,
-                           table_pages):
+                           table_pages, planes=1):
     """Norm, rotation, cache write and attention of one request cut at ``cuts``; pages in the
-    order ``table_pages``."""
+    order ``table_pages``; the values in ``planes`` planes, each attended to by itself."""
     T = qkv.shape[0]
-    kc, vc = attention_setup(ops, T + 64, nkv, d, dv, page, dtype)
+    kc, vc = attention_setup(ops, T + 64, nkv, d, dv, page, dtype, planes)
     table = torch.zeros(2, len(table_pages), dtype=torch.int32, device=DEV)
     table[1] = torch.tensor(table_pages, dtype=torch.int32)
     inv_freq = torch.tensor(freqs, dtype=torch.float32, device=DEV)
@@ -296,10 +297,20 @@ def run_attention_in_steps(ops, qkv, cuts, nh, nkv, d, dv, scale, freqs, interle
                                   kv_slot=kv_slot, nh=nh, nkv=nkv, d=d, dv=dv,
                                   q_gain=None if gains is None else gains[0].to(DEV),
                                   k_gain=None if gains is None else gains[1].to(DEV), eps=eps)
-        out = torch.empty(total, nh * dv, dtype=dtype, device=DEV)
-        ops.paged_attention(out, rows, kc, vc, table=table, positions=batch["positions"],
-                            token_req=batch["token_req"], slots=batch["slots"], nh=nh, nkv=nkv, d=d, dv=dv,
-                            scale=scale)
+        if planes == 1:
+            out = torch.empty(total, nh * dv, dtype=dtype, device=DEV)
+            ops.paged_attention(out, rows, kc, vc, table=table, positions=batch["positions"],
+                                token_req=batch["token_req"], slots=batch["slots"], nh=nh, nkv=nkv, d=d, dv=dv,
+                                scale=scale)
+        else:
+            per = []
+            for plane in vc:
+                o = torch.empty(total, nh * dv // planes, dtype=dtype, device=DEV)
+                ops.paged_attention(o, rows, kc, plane, table=table, positions=batch["positions"],
+                                    token_req=batch["token_req"], slots=batch["slots"], nh=nh, nkv=nkv, d=d,
+                                    dv=dv // planes, scale=scale)
+                per.append(o.view(total, nh, 1, dv // planes))
+            out = torch.cat(per, dim=2).reshape(total, nh * dv)
         outs.append(out.float().cpu())
         start += n
     return torch.cat(outs)
@@ -333,6 +344,20 @@ def test_attention_with_head_norm_rotation_and_value_size(ops, nh, nkv, d, dv, r
     for cuts in ([T], [20] + [1] * 25, [3, 5, 8, 2, 2, 9, 16]):
         got = run_attention_in_steps(ops, qkv, cuts, nh, nkv, d, dv, 0.3, freqs, True, gains, 1e-5, page, dtype, pages)
         close(got, want, 2e-5 if dtype == torch.float32 else 3e-2, 1e-4 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("planes", [2, 3])
+def test_values_kept_in_several_planes(ops, planes):
+    """Element i of a value head lies in plane i / (dv / planes): attending to each plane by
+    itself and laying the results side by side within every head gives the whole."""
+    T, nh, nkv, d, page = 37, 4, 2, 16, 8
+    dv = planes * d
+    qkv = rnd(T, (nh + nkv) * d + nkv * dv, seed=planes)
+    want = plain_attention(qkv.double(), nh, nkv, d, dv, 0.25, [], None, 0.0)
+    for cuts in ([T], [9, 1, 1, 2, 24]):
+        got = run_attention_in_steps(ops, qkv, cuts, nh, nkv, d, dv, 0.25, [], True, None, 0.0, page, torch.float32,
+                                     [3, 1, 4, 2, 6, 5], planes=planes)
+        close(got, want, 2e-5, 1e-4)
 
 
 @pytest.mark.parametrize("far", [0, 1, 7, 8, 15, 16, 17, 250])
