@@ -213,7 +213,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
   const float* cs = cos_tab + static_cast<int64_t>(t) * half;
   const float* sn = sin_tab + static_cast<int64_t>(t) * half;
 
-  for (int head_base = 0; head_base < nh + nkv; head_base += 4) {  // every wave the same count
+  // blockIdx.y deals the heads out four at a time (a wave each); the block with y = 0 also
+  // copies the values
+  for (int head_base = 4 * blockIdx.y; head_base < nh + nkv; head_base += 4 * gridDim.y) {
     const bool live = head_base + wave < nh + nkv;
     const int head = live ? head_base + wave : 0;
     T* hp = row + static_cast<int64_t>(head) * d;
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     }
     __syncthreads();
   }
-  if (!store_kv) return;
+  if (!store_kv || blockIdx.y != 0) return;
   // element i of a value head goes to plane i / v_chunk, V[page, kv head, i % v_chunk, offset]
   const T* vrow = row + static_cast<int64_t>(nh + nkv) * d;
   const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * v_chunk + off;
@@ -298,10 +300,14 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
     return kvc_fail("kvc_qk_norm_rope_kv_write: one to four value planes that divide the value size");
   if (T == 0) return 0;
   const int v_chunk = dv / num_v_planes;
+  // few tokens: a block per four heads, so that the launch has blocks enough; many tokens: a
+  // block per token walks the heads
+  const int all_groups = (nh + nkv + 3) / 4;
+  const int head_groups = T >= 512 ? 1 : (all_groups < 16 ? all_groups : 16);
   KVC_DISPATCH_DTYPE(
       dtype, Tp, ValuePlanes<Tp> planes{};
       for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
-      hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<Tp>, dim3(T), dim3(256), 0,
+      hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<Tp>, dim3(T, head_groups), dim3(256), 0,
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
                          static_cast<Tp*>(k_cache), planes, v_chunk, q_gain, k_gain, eps,
                          cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,

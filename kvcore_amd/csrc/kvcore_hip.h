@@ -170,11 +170,17 @@ int kvc_rglru_gates(float* a_out, float* drive, const float* u, const float* wa,
                     const float* ba, const float* bi, const float* lam, float c_decay, int T, int W,
                     int nb, kvc_stream stream);
 // S_t = a_t S_(t-1) + drive_t per channel along each request (state [slots, W] float32);
-// out[t] = S_t * gelu_tanh(y[t]).
+// out[t] = S_t * gelu_tanh(y[t]).  max_query_len bounds the tokens of a request in this step;
+// with a workspace of R * (ceil(max_query_len / kvc_rglru_scan_segment()) + 1) * 2 * W floats,
+// requests longer than a segment are scanned segment by segment side by side (two kernels: the
+// segments' sums, then the results); without one, or for short portions, one thread walks a
+// request's tokens for each channel.
+int kvc_rglru_scan_segment(void);
 int kvc_rglru_scan(void* out, int out_dtype, const float* a, const float* drive, const void* y,
                    int64_t y_stride, int y_dtype, float* state, const int32_t* positions,
                    const int32_t* token_req, const int32_t* q_start, const int32_t* slots, int R,
-                   int W, kvc_stream stream);
+                   int W, int max_query_len, float* workspace, int64_t workspace_floats,
+                   kvc_stream stream);
 // State-space recurrence with a scalar decay per head: xbc [T, >= nh*P + 2*G*N] float32 rows
 // hold x (nh heads of P), then B and C (G groups of N); per head h of group h / (nh / G):
 // dt = softplus(dt_raw[t, h] + dt_bias[h]); S = exp(-exp(a_log[h]) dt) S + dt B x^T (S [N, P],

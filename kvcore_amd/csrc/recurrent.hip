@@ -90,13 +90,18 @@ __global__ __launch_bounds__(256) void conv_state_kernel(
 // -expm1(2 log a).  A block of 256 threads owns 16 tokens x 64 outputs of one channel block
 // and walks the inputs 32 at a time through LDS; each thread sums two dot products for four
 // tokens in the order k = 0, 1, ...
-constexpr int GT = 16, GO = 64, GK = 32;
+constexpr int GT = 16, GK = 32;
 
+// GO outputs a block and TPT = GO / 16 tokens a thread: 64 and 4 for many tokens; 16 and 1 for
+// steps of few tokens, whose blocks are then four times as many (the weights, read once, are
+// all the work there, and a launch of a few dozen blocks leaves most of the chip idle).
+template <int GO, int TPT>
 __global__ __launch_bounds__(256) void rglru_gates_kernel(
     float* __restrict__ a_out, float* __restrict__ drive, const float* __restrict__ u,
     const float* __restrict__ wa, const float* __restrict__ wi, const float* __restrict__ ba,
     const float* __restrict__ bi, const float* __restrict__ lam, float c_decay, int T, int W,
     int bw, int out_tiles) {
+  static_assert(GO * (GT / TPT) == 256, "a thread per (output, group of tokens)");
   __shared__ float wa_s[GO][GK + 1];
   __shared__ float wi_s[GO][GK + 1];
   __shared__ float u_s[GT][GK];
@@ -104,11 +109,13 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   const int t0 = blockIdx.x * GT;
   const int blk = blockIdx.y / out_tiles;
   const int o0 = (blockIdx.y - blk * out_tiles) * GO;
-  const int ol = tid & (GO - 1);
-  const int tg = tid >> 6;
+  const int ol = tid % GO;
+  const int tg = tid / GO;
   const float* wa_b = wa + static_cast<int64_t>(blk) * bw * bw;
   const float* wi_b = wi + static_cast<int64_t>(blk) * bw * bw;
-  float acc_a[4] = {0.f, 0.f, 0.f, 0.f}, acc_i[4] = {0.f, 0.f, 0.f, 0.f};
+  float acc_a[TPT], acc_i[TPT];
+#pragma unroll
+  for (int tt = 0; tt < TPT; ++tt) acc_a[tt] = acc_i[tt] = 0.f;
   for (int k0 = 0; k0 < bw; k0 += GK) {
     for (int idx = tid; idx < GO * GK; idx += 256) {
       const int row = idx / GK, col = idx - row * GK;
@@ -127,8 +134,8 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
     for (int k = 0; k < GK; ++k) {
       const float va = wa_s[ol][k], vi = wi_s[ol][k];
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const float uv = u_s[tg * 4 + tt][k];
+      for (int tt = 0; tt < TPT; ++tt) {
+        const float uv = u_s[tg * TPT + tt][k];
         acc_a[tt] = fmaf(va, uv, acc_a[tt]);
         acc_i[tt] = fmaf(vi, uv, acc_i[tt]);
       }
@@ -140,8 +147,8 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   const float sp = softplus_f(lam[c]);
   const float b_a = ba[c], b_i = bi[c];
 #pragma unroll
-  for (int tt = 0; tt < 4; ++tt) {
-    const int t = t0 + tg * 4 + tt;
+  for (int tt = 0; tt < TPT; ++tt) {
+    const int t = t0 + tg * TPT + tt;
     if (t >= T) continue;
     const float r = sigmoid_f(acc_a[tt] + b_a);
     const float g = sigmoid_f(acc_i[tt] + b_i);
@@ -178,6 +185,69 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(
     out[at] = from_float<TO>(s * gelu_tanh_f(to_float(y[static_cast<int64_t>(t) * y_stride + c])));
   }
   *st = s;
+}
+
+// The same scan for long portions, cut into segments of 64 tokens so that a request's tokens are
+// worked on side by side: the first kernel scans every segment from zero and leaves its decay
+// product and its end value (and the request's state before the step); the second starts every
+// segment from what the segments before it add up to, in their order, and writes the results.
+constexpr int kScanSegment = 64;
+
+__global__ __launch_bounds__(256) void rglru_segment_sums_kernel(
+    float* __restrict__ ws, const float* __restrict__ a, const float* __restrict__ drive,
+    const float* __restrict__ state, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ token_req, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ slots, int W, int segs) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int r = blockIdx.x / segs, sg = blockIdx.x - r * segs;
+  if (c >= W) return;
+  const int b = q_start[r], e = q_start[r + 1];
+  const int t0 = b + sg * kScanSegment;
+  if (t0 >= e || token_req[b] < 0) return;
+  const int t1 = (t0 + kScanSegment < e) ? t0 + kScanSegment : e;
+  float* out = ws + (static_cast<int64_t>(r) * (segs + 1) + sg) * 2 * W + c;
+  if (sg == 0)  // the state before the step, where the second kernel finds it
+    ws[(static_cast<int64_t>(r) * (segs + 1) + segs) * 2 * W + c] =
+        positions[b] == 0 ? 0.f : state[static_cast<int64_t>(slots[r]) * W + c];
+  float prod = 1.f, end = 0.f;
+#pragma unroll 8
+  for (int t = t0; t < t1; ++t) {
+    const int64_t at = static_cast<int64_t>(t) * W + c;
+    const float av = a[at];
+    prod *= av;
+    end = fmaf(av, end, drive[at]);
+  }
+  out[0] = prod;
+  out[W] = end;
+}
+
+template <typename TY, typename TO>
+__global__ __launch_bounds__(256) void rglru_scan_segments_kernel(
+    TO* __restrict__ out, const float* __restrict__ a, const float* __restrict__ drive,
+    const TY* __restrict__ y, int64_t y_stride, float* __restrict__ state,
+    const float* __restrict__ ws, const int32_t* __restrict__ token_req,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int W, int segs) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int r = blockIdx.x / segs, sg = blockIdx.x - r * segs;
+  if (c >= W) return;
+  const int b = q_start[r], e = q_start[r + 1];
+  const int t0 = b + sg * kScanSegment;
+  if (t0 >= e) return;
+  const int t1 = (t0 + kScanSegment < e) ? t0 + kScanSegment : e;
+  if (token_req[b] < 0) {
+    for (int t = t0; t < t1; ++t) out[static_cast<int64_t>(t) * W + c] = from_float<TO>(0.f);
+    return;
+  }
+  const float* sums = ws + static_cast<int64_t>(r) * (segs + 1) * 2 * W + c;
+  float s = sums[static_cast<int64_t>(segs) * 2 * W];
+  for (int j = 0; j < sg; ++j) s = fmaf(sums[static_cast<int64_t>(j) * 2 * W], s, sums[static_cast<int64_t>(j) * 2 * W + W]);
+#pragma unroll 8
+  for (int t = t0; t < t1; ++t) {
+    const int64_t at = static_cast<int64_t>(t) * W + c;
+    s = fmaf(a[at], s, drive[at]);
+    out[at] = from_float<TO>(s * gelu_tanh_f(to_float(y[static_cast<int64_t>(t) * y_stride + c])));
+  }
+  if (t1 == e) state[static_cast<int64_t>(slots[r]) * W + c] = s;
 }
 
 // ------------------------------------------------------ state-space recurrence
@@ -287,6 +357,144 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   }
 }
 
+// The same recurrence for heads of 64 value channels and more (blocks of 256 threads), made for
+// long portions: thread (pl, ns) keeps S[n, p0 + pl] for the NPT consecutive rows n = ns * NPT ..
+// in registers; B and C lie in LDS padded with zeros to 4 * NPT rows, so that the inner loop has
+// no bounds and reads them 16 bytes at a time; and while a stage of 16 tokens is worked on, the
+// next stage's B, C, x and step sizes are already on their way from memory into registers (a
+// block has one wave a SIMD and nothing else to hide that latency behind).
+template <int NPT, typename TD>
+__global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
+    float* __restrict__ y, const float* __restrict__ xbc, int64_t xbc_stride,
+    const TD* __restrict__ dt_raw, int64_t dt_stride, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int P, int N,
+    int G) {
+  constexpr int PT = 64;
+  constexpr int NP = NS * NPT;             // padded rows of the state
+  constexpr int NB = SC * NP / 256;        // values of B (and of C) a thread fetches per stage
+  constexpr int NX = SC * PT / 256;
+  __shared__ __attribute__((aligned(16))) float b_s[SC * NP];
+  __shared__ __attribute__((aligned(16))) float c_s[SC * NP];
+  __shared__ float x_s[SC * PT];
+  __shared__ float y_s[SC * NS * PT];
+  __shared__ float dt_s[SC];
+  __shared__ float dec_s[SC];
+  const int r = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PT;
+  const int tid = threadIdx.x;
+  const int pl = tid & (PT - 1), ns = tid >> 6;
+  const int p = p0 + pl;
+  const bool p_ok = p < P;
+  const int inner = nh * P;
+  const int b = q_start[r], e = q_start[r + 1];
+  if (e <= b) return;
+  if (token_req[b] < 0) {
+    for (int idx = tid; idx < (e - b) * PT; idx += 256) {
+      const int tt = idx / PT, q = p0 + idx - tt * PT;
+      if (q < P) y[static_cast<int64_t>(b + tt) * inner + h * P + q] = 0.f;
+    }
+    return;
+  }
+  const int g = h / (nh / G);
+  float* st = state + (static_cast<int64_t>(slots[r]) * nh + h) * N * P;
+  const bool fresh = positions[b] == 0;
+  float s[NPT];
+#pragma unroll
+  for (int k = 0; k < NPT; ++k) {
+    const int n = ns * NPT + k;
+    s[k] = (!fresh && p_ok && n < N) ? st[static_cast<int64_t>(n) * P + p] : 0.f;
+  }
+  const float neg_a = -expf(a_log[h]);
+  const float bias = dt_bias[h];
+  const float skip = d_skip[h];
+  const int off_b = inner + g * N, off_c = inner + G * N + g * N;
+
+  float rb[NB], rc[NB], rx[NX], rdt = 0.f;
+  auto fetch = [&](int c0) {  // the stage that starts at token c0, into registers
+    const int nt = (e - c0 < SC) ? e - c0 : SC;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int idx = tid + i * 256;
+      const int tt = idx / NP, n = idx - tt * NP;
+      const bool ok = tt < nt && n < N;
+      const float* row = xbc + static_cast<int64_t>(c0 + (ok ? tt : 0)) * xbc_stride;
+      rb[i] = ok ? row[off_b + n] : 0.f;
+      rc[i] = ok ? row[off_c + n] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < NX; ++i) {
+      const int idx = tid + i * 256;
+      const int tt = idx / PT, q = idx - tt * PT;
+      const bool ok = tt < nt && p0 + q < P;
+      rx[i] = ok ? xbc[static_cast<int64_t>(c0 + tt) * xbc_stride + h * P + p0 + q] : 0.f;
+    }
+    rdt = tid < nt ? to_float(dt_raw[static_cast<int64_t>(c0 + tid) * dt_stride + h]) : 0.f;
+  };
+  auto stash = [&]() {  // registers to LDS
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      b_s[tid + i * 256] = rb[i];
+      c_s[tid + i * 256] = rc[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NX; ++i) x_s[tid + i * 256] = rx[i];
+    if (tid < SC) {
+      const float dt = softplus_f(rdt + bias);
+      dt_s[tid] = dt;
+      dec_s[tid] = expf(neg_a * dt);
+    }
+  };
+  fetch(b);
+  stash();
+  __syncthreads();
+  for (int c0 = b; c0 < e; c0 += SC) {
+    const int nt = (e - c0 < SC) ? e - c0 : SC;
+    const bool more = c0 + SC < e;
+    if (more) fetch(c0 + SC);
+    for (int tt = 0; tt < nt; ++tt) {
+      const float dec = dec_s[tt];
+      const float xv = x_s[tt * PT + pl] * dt_s[tt];
+      const float4* bt = reinterpret_cast<const float4*>(b_s + tt * NP + ns * NPT);
+      const float4* ct = reinterpret_cast<const float4*>(c_s + tt * NP + ns * NPT);
+      float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int k4 = 0; k4 < NPT / 4; ++k4) {
+        const float4 bv = bt[k4], cv = ct[k4];
+        s[4 * k4 + 0] = fmaf(dec, s[4 * k4 + 0], bv.x * xv);
+        s[4 * k4 + 1] = fmaf(dec, s[4 * k4 + 1], bv.y * xv);
+        s[4 * k4 + 2] = fmaf(dec, s[4 * k4 + 2], bv.z * xv);
+        s[4 * k4 + 3] = fmaf(dec, s[4 * k4 + 3], bv.w * xv);
+        acc0 = fmaf(s[4 * k4 + 0], cv.x, acc0);
+        acc1 = fmaf(s[4 * k4 + 1], cv.y, acc1);
+        acc0 = fmaf(s[4 * k4 + 2], cv.z, acc0);
+        acc1 = fmaf(s[4 * k4 + 3], cv.w, acc1);
+      }
+      y_s[(tt * NS + ns) * PT + pl] = acc0 + acc1;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nt * PT; idx += 256) {
+      const int tt = idx / PT, q = idx - tt * PT;
+      if (p0 + q >= P) continue;
+      float v = 0.f;
+#pragma unroll
+      for (int z = 0; z < NS; ++z) v += y_s[(tt * NS + z) * PT + q];
+      y[static_cast<int64_t>(c0 + tt) * inner + h * P + p0 + q] = fmaf(skip, x_s[tt * PT + q], v);
+    }
+    __syncthreads();
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+  if (!p_ok) return;
+#pragma unroll
+  for (int k = 0; k < NPT; ++k) {
+    const int n = ns * NPT + k;
+    if (n < N) st[static_cast<int64_t>(n) * P + p] = s[k];
+  }
+}
+
 // out[t, c] = gain[c] * v / sqrt(mean over c's group of v^2 + eps), v = y[t, c] * silu(z[t, c]):
 // the gate first, then the norm in `groups` equal parts.  One block per (token, part).
 template <typename TZ, typename TO>
@@ -355,23 +563,47 @@ extern "C" int kvc_rglru_gates(float* a_out, float* drive, const float* u, const
   if (T < 0 || W <= 0 || nb <= 0 || W % nb) return kvc_fail("kvc_rglru_gates: bad sizes");
   if (T == 0) return 0;
   const int bw = W / nb;
-  const int out_tiles = (bw + GO - 1) / GO;
+  const bool few = T <= 2 * GT;  // few tokens: smaller tiles of outputs, four times the blocks
+  const int go = few ? 16 : 64;
+  const int out_tiles = (bw + go - 1) / go;
   const dim3 grid((T + GT - 1) / GT, nb * out_tiles);  // tokens on x, which has no 16-bit limit
   if (grid.y > 65535u) return kvc_fail("kvc_rglru_gates: too many channel tiles");
-  hipLaunchKernelGGL(rglru_gates_kernel, grid, dim3(256), 0, S(stream), a_out, drive, u, wa, wi, ba,
-                     bi, lam, c_decay, T, W, bw, out_tiles);
+  if (few)
+    hipLaunchKernelGGL((rglru_gates_kernel<16, 1>), grid, dim3(256), 0, S(stream), a_out, drive, u, wa,
+                       wi, ba, bi, lam, c_decay, T, W, bw, out_tiles);
+  else
+    hipLaunchKernelGGL((rglru_gates_kernel<64, 4>), grid, dim3(256), 0, S(stream), a_out, drive, u, wa,
+                       wi, ba, bi, lam, c_decay, T, W, bw, out_tiles);
   return kvc_check_launch("kvc_rglru_gates");
 }
+
+extern "C" int kvc_rglru_scan_segment(void) { return kScanSegment; }
 
 extern "C" int kvc_rglru_scan(void* out, int out_dtype, const float* a, const float* drive,
                               const void* y, int64_t y_stride, int y_dtype, float* state,
                               const int32_t* positions, const int32_t* token_req,
                               const int32_t* q_start, const int32_t* slots, int R, int W,
+                              int max_query_len, float* workspace, int64_t workspace_floats,
                               kvc_stream stream) {
   if (R < 0 || W <= 0 || y_stride < W) return kvc_fail("kvc_rglru_scan: bad sizes");
   if (R == 0) return 0;
-  const dim3 grid(R, (W + 255) / 256);
-  if (grid.y > 65535u) return kvc_fail("kvc_rglru_scan: too many channels for one launch");
+  const unsigned tiles = (W + 255) / 256;
+  if (tiles > 65535u) return kvc_fail("kvc_rglru_scan: too many channels for one launch");
+  const int segs = (max_query_len + kScanSegment - 1) / kScanSegment;
+  if (segs > 1 && workspace != nullptr) {
+    // long portions: segments side by side, two kernels
+    if (workspace_floats < static_cast<int64_t>(R) * (segs + 1) * 2 * W)
+      return kvc_fail("kvc_rglru_scan: the workspace is too small");
+    const dim3 grid(static_cast<unsigned>(R) * segs, tiles);
+    hipLaunchKernelGGL(rglru_segment_sums_kernel, grid, dim3(256), 0, S(stream), workspace, a, drive,
+                       state, positions, token_req, q_start, slots, W, segs);
+    KVC_DISPATCH_2(y_dtype, TY, out_dtype, TO,
+                   hipLaunchKernelGGL((rglru_scan_segments_kernel<TY, TO>), grid, dim3(256), 0, S(stream),
+                                      static_cast<TO*>(out), a, drive, static_cast<const TY*>(y),
+                                      y_stride, state, workspace, token_req, q_start, slots, W, segs));
+    return kvc_check_launch("kvc_rglru_scan (segments)");
+  }
+  const dim3 grid(R, tiles);
   KVC_DISPATCH_2(y_dtype, TY, out_dtype, TO,
                  hipLaunchKernelGGL((rglru_scan_kernel<TY, TO>), grid, dim3(256), 0, S(stream),
                                     static_cast<TO*>(out), a, drive, static_cast<const TY*>(y),
@@ -405,7 +637,22 @@ extern "C" int kvc_ssm_scan(float* y, const float* xbc, int64_t xbc_stride, cons
                                         xbc, xbc_stride, static_cast<const TD*>(dt_raw), dt_stride, \
                                         dt_bias, a_log, d_skip, state, positions, token_req,       \
                                         q_start, slots, nh, P, N, G, PT))
-  if (per_thread <= 16) {
+#define KVC_SSM_LAUNCH_WIDE(NPT)                                                                   \
+  KVC_DISPATCH_DTYPE(dt_dtype, TD,                                                                 \
+                     hipLaunchKernelGGL((ssm_scan_wide_kernel<NPT, TD>), grid, dim3(256), 0,       \
+                                        S(stream), y, xbc, xbc_stride,                             \
+                                        static_cast<const TD*>(dt_raw), dt_stride, dt_bias, a_log, \
+                                        d_skip, state, positions, token_req, q_start, slots, nh, P, \
+                                        N, G))
+  if (PT == 64) {  // heads of 64 value channels and more: the kernel made for long portions
+    if (per_thread <= 16) {
+      KVC_SSM_LAUNCH_WIDE(16);
+    } else if (per_thread <= 32) {
+      KVC_SSM_LAUNCH_WIDE(32);
+    } else {
+      KVC_SSM_LAUNCH_WIDE(64);
+    }
+  } else if (per_thread <= 16) {
     KVC_SSM_LAUNCH(16);
   } else if (per_thread <= 32) {
     KVC_SSM_LAUNCH(32);
@@ -413,6 +660,7 @@ extern "C" int kvc_ssm_scan(float* y, const float* xbc, int64_t xbc_stride, cons
     KVC_SSM_LAUNCH(64);
   }
 #undef KVC_SSM_LAUNCH
+#undef KVC_SSM_LAUNCH_WIDE
   return kvc_check_launch("kvc_ssm_scan");
 }
 

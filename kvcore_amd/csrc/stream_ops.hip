@@ -52,6 +52,51 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(T* __restrict__ out,
   }
 }
 
+// The same for rows of up to 256 * NV values, which a thread keeps in registers: residual and
+// delta are read once and everything else is arithmetic and two block sums.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void add_layernorm_regs_kernel(T* __restrict__ out,
+                                                                 float* __restrict__ residual,
+                                                                 const T* __restrict__ delta,
+                                                                 const float* __restrict__ weight,
+                                                                 const float* __restrict__ bias,
+                                                                 float eps, int H) {
+  __shared__ float scratch[16];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
+  float* r = residual + base;
+  float v[NV];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * 256;
+    v[i] = 0.f;
+    if (c < H) {
+      v[i] = r[c];
+      if (delta != nullptr) {
+        v[i] += to_float(delta[base + c]);
+        r[c] = v[i];
+      }
+      sum += v[i];
+    }
+  }
+  const float mean = block_sum(sum, scratch) / static_cast<float>(H);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < H) {
+      v[i] -= mean;
+      ss = fmaf(v[i], v[i], ss);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < H) out[base + c] = from_float<T>(fmaf(v[i] * inv, weight[c], bias != nullptr ? bias[c] : 0.f));
+  }
+}
+
 constexpr int kMaxBranches = 4;
 struct Branches {
   const float* x[kMaxBranches];
@@ -103,6 +148,20 @@ extern "C" int kvc_add_layernorm(void* out, float* residual, const void* delta, 
                                  kvc_stream stream) {
   if (T < 0 || H <= 0) return kvc_fail("kvc_add_layernorm: bad sizes");
   if (T == 0) return 0;
+  if (H <= 256 * 8) {
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((add_layernorm_regs_kernel<Tp, 8>), dim3(T), dim3(256), 0, S(stream),
+                                          static_cast<Tp*>(out), residual,
+                                          static_cast<const Tp*>(delta), weight, bias, eps, H));
+    return kvc_check_launch("kvc_add_layernorm");
+  }
+  if (H <= 256 * 32) {
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((add_layernorm_regs_kernel<Tp, 32>), dim3(T), dim3(256), 0, S(stream),
+                                          static_cast<Tp*>(out), residual,
+                                          static_cast<const Tp*>(delta), weight, bias, eps, H));
+    return kvc_check_launch("kvc_add_layernorm");
+  }
   KVC_DISPATCH_DTYPE(dtype, Tp,
                      hipLaunchKernelGGL(add_layernorm_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
                                         static_cast<Tp*>(out), residual,

@@ -54,7 +54,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_add_row": [P, P, I, I, P],
         "kvc_causal_conv": [P, L, I, P, L, I, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
         "kvc_rglru_gates": [P, P, P, P, P, P, P, P, F, I, I, I, P],
-        "kvc_rglru_scan": [P, I, P, P, P, L, I, P, P, P, P, P, I, I, P],
+        "kvc_rglru_scan": [P, I, P, P, P, L, I, P, P, P, P, P, I, I, I, P, L, P],
         "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "kvc_gated_group_rmsnorm": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
@@ -96,6 +96,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.kvc_argmax_static_capacity.argtypes = []
     lib.kvc_ssm_scan_max_state.restype = c_int
     lib.kvc_ssm_scan_max_state.argtypes = []
+    lib.kvc_rglru_scan_segment.restype = c_int
+    lib.kvc_rglru_scan_segment.argtypes = []
 
 
 def load(build_if_missing: bool = True) -> ctypes.CDLL:
@@ -1115,12 +1117,23 @@ def rglru_gates(a_out: torch.Tensor, drive: torch.Tensor, u: torch.Tensor, wa: t
                                   _dev(lam, "lam", f), float(c_decay), T, W, nb, _stream()), "kvc_rglru_gates")
 
 
+def rglru_scan_workspace_floats(num_reqs: int, width: int, max_query_len: int) -> int:
+    """float32 values of workspace with which ``rglru_scan`` works on the segments of long
+    portions side by side (0: the portions are too short to gain from it)."""
+    seg = int(load().kvc_rglru_scan_segment())
+    segs = -(-max_query_len // seg)
+    return 0 if segs <= 1 else num_reqs * (segs + 1) * 2 * width
+
+
 def rglru_scan(out: torch.Tensor, a: torch.Tensor, drive: torch.Tensor, y: torch.Tensor,
                state: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
-               q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int) -> None:
+               q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int, max_query_len: int = 0,
+               workspace: torch.Tensor | None = None) -> None:
     """``S_t = a_t S_(t-1) + drive_t`` per channel along each request, ``out[t] = S_t *
     gelu_tanh(y[t])``; ``state [slots, W]`` float32 is read (a request at position 0 starts
-    from zero) and rewritten."""
+    from zero) and rewritten.  With ``max_query_len`` (a bound on a request's tokens in this
+    step) and a float32 ``workspace`` of ``rglru_scan_workspace_floats`` values, long portions
+    are scanned in segments side by side."""
     T, W = a.shape
     if drive.shape != (T, W) or out.shape != (T, W) or not out.is_contiguous() or state.shape[1:] != (W,):
         raise KernelError("rglru_scan: shapes do not match")
@@ -1129,8 +1142,9 @@ def rglru_scan(out: torch.Tensor, a: torch.Tensor, drive: torch.Tensor, y: torch
         _dev(out, "out"), _code(out, "out"), _dev(a, "a", torch.float32), _dev(drive, "drive", torch.float32),
         y_ptr, y_stride, y_code, _dev(state, "state", torch.float32),
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, W, _stream()),
-        "kvc_rglru_scan")
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, W,
+        int(max_query_len), None if workspace is None else _dev(workspace, "workspace", torch.float32),
+        0 if workspace is None else workspace.numel(), _stream()), "kvc_rglru_scan")
 
 
 def ssm_scan_max_state() -> int:

@@ -101,7 +101,14 @@ class GatedLinearRecurrence(Mixer):
         ops.rglru_gates(a, drive, u, p["gate_a.weight"], p["gate_i.weight"], p["gate_a.bias"],
                         p["gate_i.bias"], p["lam"], self.decay_scale)
         gated = ctx.buf(f"lru_gated:{W}", W)
-        ops.rglru_scan(gated, a, drive, yx[:, :W], lru_state, **batch)
+        # long portions are scanned in segments side by side, which takes a workspace
+        need = ops.rglru_scan_workspace_floats(ctx.num_reqs, W, ctx.max_query_len)
+        workspace = None
+        if need:  # rows of 2 W sums; the buffer only ever grows, to the largest step seen
+            workspace = ctx.buffers.get(f"lru_scan_sums:{W}", need // (2 * W), 2 * W, torch.float32,
+                                        reserve=ctx.buffers.token_capacity // 32 + 2 * ctx.buffers.seq_capacity)
+        ops.rglru_scan(gated, a, drive, yx[:, :W], lru_state, max_query_len=ctx.max_query_len,
+                       workspace=workspace, **batch)
         if self.float32_result:
             out = ctx.buf("mixer_out_f32_b", self.hidden_size, torch.float32)
         else:

@@ -191,6 +191,43 @@ def test_gated_linear_recurrence_whole_and_in_steps(ops, W, nb):
         close(state[2], last, 2e-5, 2e-5)
 
 
+def test_long_portions_are_scanned_in_segments_side_by_side(ops):
+    """With a workspace, requests longer than a segment are cut into segments that are scanned
+    side by side and joined in order: the same results, whatever the portions, beside short
+    requests and a padded one, from a state that an earlier step left."""
+    T, W, nb = 333, 96, 2
+    bw = W // nb
+    u, y = rnd(T, W, seed=1), rnd(T, W, seed=2)
+    wa, wi = rnd(nb, bw, bw, seed=3, std=0.5), rnd(nb, bw, bw, seed=4, std=0.5)
+    ba, bi = rnd(nb, bw, seed=5), rnd(nb, bw, seed=6)
+    lam = rnd(W, seed=7) * 2 - 3
+    want, last = plain_recurrence(*(t.double() for t in (u, y, wa, wi, ba, bi, lam)), 8.0)
+    d = [t.to(DEV) for t in (wa, wi, ba, bi, lam)]
+    for cuts in ([T], [64, 65, 1, 129, 74], [200, 133], [3, 330]):
+        state = torch.full((4, W), float("nan"), device=DEV)
+        outs, start = [], 0
+        for n in cuts:
+            batch, total = batch_tensors([(3, 5, 2), (2, start, n), None, (0, 0, 70)])
+            uu = torch.zeros(total, W)
+            yy = torch.zeros(total, W)
+            uu[2: 2 + n], yy[2: 2 + n] = u[start: start + n], y[start: start + n]
+            uu[3 + n:], yy[3 + n:] = u[:70], y[:70]  # a second request: the first 70 tokens again
+            state[3] = 0.5
+            a = torch.empty(total, W, device=DEV)
+            drive = torch.empty(total, W, device=DEV)
+            ops.rglru_gates(a, drive, uu.to(DEV), *d, 8.0)
+            out = torch.empty(total, W, device=DEV)
+            longest = max(n, 70)
+            ws = torch.full((ops.rglru_scan_workspace_floats(4, W, longest),), float("nan"), device=DEV)
+            ops.rglru_scan(out, a, drive, yy.to(DEV), state, max_query_len=longest, workspace=ws, **batch)
+            outs.append(out[2: 2 + n].cpu())
+            close(out[3 + n:], want[:70], 2e-5, 2e-5)
+            assert torch.equal(out[2 + n].cpu(), torch.zeros(W))
+            start += n
+        close(torch.cat(outs), want, 2e-5, 2e-5)
+        close(state[2], last, 2e-5, 2e-5)
+
+
 def test_recurrence_keeps_a_far_token(ops):
     """A channel whose decay is almost 1 still carries its first input after 600 tokens, through
     steps of every size; a channel whose decay is almost 0 carries nothing."""
