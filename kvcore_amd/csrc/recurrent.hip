@@ -357,13 +357,14 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(
   }
 }
 
-// The same recurrence for heads of 64 value channels and more (blocks of 256 threads), made for
+// The same recurrence for heads of 16 value channels and more (blocks of 256 threads over PT = 64
+// or 16 of them; the narrow tiles where the wide ones would leave compute units idle), made for
 // long portions: thread (pl, ns) keeps S[n, p0 + pl] for the NPT consecutive rows n = ns * NPT ..
 // in registers; B and C lie in LDS padded with zeros to 4 * NPT rows, so that the inner loop has
 // no bounds and reads them 16 bytes at a time; and while a stage of 16 tokens is worked on, the
 // next stage's B, C, x and step sizes are already on their way from memory into registers (a
 // block has one wave a SIMD and nothing else to hide that latency behind).
-template <int NPT, typename TD>
+template <int NPT, int PT, typename TD>
 __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
     float* __restrict__ y, const float* __restrict__ xbc, int64_t xbc_stride,
     const TD* __restrict__ dt_raw, int64_t dt_stride, const float* __restrict__ dt_bias,
@@ -371,19 +372,20 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int P, int N,
     int G) {
-  constexpr int PT = 64;
-  constexpr int NP = NS * NPT;             // padded rows of the state
+  constexpr int NSL = 256 / PT;            // threads that share a column of the state
+  constexpr int NP = NSL * NPT;            // padded rows of the state
   constexpr int NB = SC * NP / 256;        // values of B (and of C) a thread fetches per stage
-  constexpr int NX = SC * PT / 256;
+  constexpr int NX = (SC * PT + 255) / 256;
+  static_assert(NPT % 4 == 0 && (SC * NP) % 256 == 0, "whole 16-byte reads and whole fetch rounds");
   __shared__ __attribute__((aligned(16))) float b_s[SC * NP];
   __shared__ __attribute__((aligned(16))) float c_s[SC * NP];
   __shared__ float x_s[SC * PT];
-  __shared__ float y_s[SC * NS * PT];
+  __shared__ float y_s[SC * NSL * PT];
   __shared__ float dt_s[SC];
   __shared__ float dec_s[SC];
   const int r = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PT;
   const int tid = threadIdx.x;
-  const int pl = tid & (PT - 1), ns = tid >> 6;
+  const int pl = tid % PT, ns = tid / PT;
   const int p = p0 + pl;
   const bool p_ok = p < P;
   const int inner = nh * P;
@@ -426,7 +428,7 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
     for (int i = 0; i < NX; ++i) {
       const int idx = tid + i * 256;
       const int tt = idx / PT, q = idx - tt * PT;
-      const bool ok = tt < nt && p0 + q < P;
+      const bool ok = idx < SC * PT && tt < nt && p0 + q < P;
       rx[i] = ok ? xbc[static_cast<int64_t>(c0 + tt) * xbc_stride + h * P + p0 + q] : 0.f;
     }
     rdt = tid < nt ? to_float(dt_raw[static_cast<int64_t>(c0 + tid) * dt_stride + h]) : 0.f;
@@ -438,7 +440,8 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
       c_s[tid + i * 256] = rc[i];
     }
 #pragma unroll
-    for (int i = 0; i < NX; ++i) x_s[tid + i * 256] = rx[i];
+    for (int i = 0; i < NX; ++i)
+      if (tid + i * 256 < SC * PT) x_s[tid + i * 256] = rx[i];
     if (tid < SC) {
       const float dt = softplus_f(rdt + bias);
       dt_s[tid] = dt;
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
         acc0 = fmaf(s[4 * k4 + 2], cv.z, acc0);
         acc1 = fmaf(s[4 * k4 + 3], cv.w, acc1);
       }
-      y_s[(tt * NS + ns) * PT + pl] = acc0 + acc1;
+      y_s[(tt * NSL + ns) * PT + pl] = acc0 + acc1;
     }
     __syncthreads();
     for (int idx = tid; idx < nt * PT; idx += 256) {
@@ -478,7 +481,7 @@ __global__ __launch_bounds__(256) void ssm_scan_wide_kernel(
       if (p0 + q >= P) continue;
       float v = 0.f;
 #pragma unroll
-      for (int z = 0; z < NS; ++z) v += y_s[(tt * NS + z) * PT + q];
+      for (int z = 0; z < NSL; ++z) v += y_s[(tt * NSL + z) * PT + q];
       y[static_cast<int64_t>(c0 + tt) * inner + h * P + p0 + q] = fmaf(skip, x_s[tt * PT + q], v);
     }
     __syncthreads();
@@ -637,20 +640,32 @@ extern "C" int kvc_ssm_scan(float* y, const float* xbc, int64_t xbc_stride, cons
                                         xbc, xbc_stride, static_cast<const TD*>(dt_raw), dt_stride, \
                                         dt_bias, a_log, d_skip, state, positions, token_req,       \
                                         q_start, slots, nh, P, N, G, PT))
-#define KVC_SSM_LAUNCH_WIDE(NPT)                                                                   \
+#define KVC_SSM_LAUNCH_WIDE(NPT, PTW)                                                              \
   KVC_DISPATCH_DTYPE(dt_dtype, TD,                                                                 \
-                     hipLaunchKernelGGL((ssm_scan_wide_kernel<NPT, TD>), grid, dim3(256), 0,       \
-                                        S(stream), y, xbc, xbc_stride,                             \
-                                        static_cast<const TD*>(dt_raw), dt_stride, dt_bias, a_log, \
-                                        d_skip, state, positions, token_req, q_start, slots, nh, P, \
-                                        N, G))
-  if (PT == 64) {  // heads of 64 value channels and more: the kernel made for long portions
-    if (per_thread <= 16) {
-      KVC_SSM_LAUNCH_WIDE(16);
-    } else if (per_thread <= 32) {
-      KVC_SSM_LAUNCH_WIDE(32);
+                     hipLaunchKernelGGL((ssm_scan_wide_kernel<NPT, PTW, TD>),                      \
+                                        dim3(R, nh, (P + PTW - 1) / PTW), dim3(256), 0, S(stream), \
+                                        y, xbc, xbc_stride, static_cast<const TD*>(dt_raw),        \
+                                        dt_stride, dt_bias, a_log, d_skip, state, positions,       \
+                                        token_req, q_start, slots, nh, P, N, G))
+  // tiles of 16 value channels (sixteen threads a column of the state) where tiles of 64 would
+  // give fewer blocks than the chip has compute units
+  const int64_t wide_blocks = static_cast<int64_t>(R) * nh * ((P + 63) / 64);
+  if (P >= 16 && (P < 64 || wide_blocks < kvc_device_compute_units())) {
+    const int rows = (N + 15) / 16;
+    if (rows <= 4) {
+      KVC_SSM_LAUNCH_WIDE(4, 16);
+    } else if (rows <= 8) {
+      KVC_SSM_LAUNCH_WIDE(8, 16);
     } else {
-      KVC_SSM_LAUNCH_WIDE(64);
+      KVC_SSM_LAUNCH_WIDE(16, 16);
+    }
+  } else if (PT == 64) {  // heads of 64 value channels and more
+    if (per_thread <= 16) {
+      KVC_SSM_LAUNCH_WIDE(16, 64);
+    } else if (per_thread <= 32) {
+      KVC_SSM_LAUNCH_WIDE(32, 64);
+    } else {
+      KVC_SSM_LAUNCH_WIDE(64, 64);
     }
   } else if (per_thread <= 16) {
     KVC_SSM_LAUNCH(16);

@@ -64,14 +64,16 @@ __global__ __launch_bounds__(256) void add_layernorm_regs_kernel(T* __restrict__
   __shared__ float scratch[16];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
   float* r = residual + base;
-  float v[NV];
+  float v[NV], w[NV], sh[NV];  // gain and shift come with the row: one trip to memory in all
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int c = threadIdx.x + i * 256;
-    v[i] = 0.f;
+    v[i] = w[i] = sh[i] = 0.f;
     if (c < H) {
       v[i] = r[c];
+      w[i] = weight[c];
+      if (bias != nullptr) sh[i] = bias[c];
       if (delta != nullptr) {
         v[i] += to_float(delta[base + c]);
         r[c] = v[i];
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(256) void add_layernorm_regs_kernel(T* __restrict__
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int c = threadIdx.x + i * 256;
-    if (c < H) out[base + c] = from_float<T>(fmaf(v[i] * inv, weight[c], bias != nullptr ? bias[c] : 0.f));
+    if (c < H) out[base + c] = from_float<T>(fmaf(v[i] * inv, w[i], sh[i]));
   }
 }
 
@@ -104,23 +106,58 @@ struct Branches {
 };
 
 // out[t] = (1 / n) * sum_b gain_b * x_b[t] / sqrt(mean(x_b[t]^2) + eps).  One block per row.
-template <typename T>
+// REGS: the rows (up to 256 * 8 values) and the gains are fetched once, all at the start, and
+// kept in registers; otherwise a row is read twice.
+template <typename T, bool REGS>
 __global__ __launch_bounds__(256) void rms_branches_mean_kernel(T* __restrict__ out, Branches br,
                                                                 int n, float eps, int H) {
   __shared__ float scratch[16];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
-  float inv[kMaxBranches];
-  for (int b = 0; b < n; ++b) {
-    const float* x = br.x[b] + base;
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) ss = fmaf(x[i], x[i], ss);
-    inv[b] = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(H) + eps);
-  }
   const float share = 1.f / static_cast<float>(n);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float acc = 0.f;
-    for (int b = 0; b < n; ++b) acc = fmaf(br.x[b][base + i] * inv[b], br.gain[b][i], acc);
-    out[base + i] = from_float<T>(acc * share);
+  if constexpr (REGS) {
+    constexpr int NV = 8;
+    float x[kMaxBranches][NV], gn[kMaxBranches][NV], ss[kMaxBranches];
+#pragma unroll
+    for (int b = 0; b < kMaxBranches; ++b) {
+      ss[b] = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * 256;
+        const bool ok = b < n && c < H;
+        x[b][i] = ok ? br.x[b][base + c] : 0.f;
+        gn[b][i] = ok ? br.gain[b][c] : 0.f;
+        ss[b] = fmaf(x[b][i], x[b][i], ss[b]);
+      }
+    }
+    float acc[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int b = 0; b < kMaxBranches; ++b) {
+      if (b < n) {  // uniform
+        const float inv = 1.f / sqrtf(block_sum(ss[b], scratch) / static_cast<float>(H) + eps);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) acc[i] = fmaf(x[b][i] * inv, gn[b][i], acc[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = threadIdx.x + i * 256;
+      if (c < H) out[base + c] = from_float<T>(acc[i] * share);
+    }
+  } else {
+    float inv[kMaxBranches];
+    for (int b = 0; b < n; ++b) {
+      const float* x = br.x[b] + base;
+      float ss = 0.f;
+      for (int i = threadIdx.x; i < H; i += blockDim.x) ss = fmaf(x[i], x[i], ss);
+      inv[b] = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(H) + eps);
+    }
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float acc = 0.f;
+      for (int b = 0; b < n; ++b) acc = fmaf(br.x[b][base + i] * inv[b], br.gain[b][i], acc);
+      out[base + i] = from_float<T>(acc * share);
+    }
   }
 }
 
@@ -180,9 +217,14 @@ extern "C" int kvc_rms_branches_mean(void* out, const float* const* host_x,
     br.x[b] = host_x[b];
     br.gain[b] = host_gain[b];
   }
-  KVC_DISPATCH_DTYPE(dtype, Tp,
-                     hipLaunchKernelGGL(rms_branches_mean_kernel<Tp>, dim3(T), dim3(256), 0,
-                                        S(stream), static_cast<Tp*>(out), br, n, eps, H));
+  if (H <= 256 * 8)
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((rms_branches_mean_kernel<Tp, true>), dim3(T), dim3(256), 0,
+                                          S(stream), static_cast<Tp*>(out), br, n, eps, H));
+  else
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((rms_branches_mean_kernel<Tp, false>), dim3(T), dim3(256), 0,
+                                          S(stream), static_cast<Tp*>(out), br, n, eps, H));
   return kvc_check_launch("kvc_rms_branches_mean");
 }
 
