@@ -116,20 +116,42 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   float acc_a[TPT], acc_i[TPT];
 #pragma unroll
   for (int tt = 0; tt < TPT; ++tt) acc_a[tt] = acc_i[tt] = 0.f;
-  for (int k0 = 0; k0 < bw; k0 += GK) {
-    for (int idx = tid; idx < GO * GK; idx += 256) {
+  // a stage of 32 inputs is fetched into registers while the stage before it is multiplied
+  constexpr int NW = GO * GK / 256, NU = GT * GK / 256;
+  float wa_r[NW], wi_r[NW], u_r[NU];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int idx = tid + i * 256;
       const int row = idx / GK, col = idx - row * GK;
       const bool ok = o0 + row < bw && k0 + col < bw;
       const int64_t off = static_cast<int64_t>(o0 + row) * bw + k0 + col;
-      wa_s[row][col] = ok ? wa_b[off] : 0.f;
-      wi_s[row][col] = ok ? wi_b[off] : 0.f;
+      wa_r[i] = ok ? wa_b[off] : 0.f;
+      wi_r[i] = ok ? wi_b[off] : 0.f;
     }
-    for (int idx = tid; idx < GT * GK; idx += 256) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int idx = tid + i * 256;
       const int row = idx / GK, col = idx - row * GK;
       const bool ok = t0 + row < T && k0 + col < bw;
-      u_s[row][col] = ok ? u[static_cast<int64_t>(t0 + row) * W + blk * bw + k0 + col] : 0.f;
+      u_r[i] = ok ? u[static_cast<int64_t>(t0 + row) * W + blk * bw + k0 + col] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < bw; k0 += GK) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int idx = tid + i * 256;
+      wa_s[idx / GK][idx % GK] = wa_r[i];
+      wi_s[idx / GK][idx % GK] = wi_r[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int idx = tid + i * 256;
+      u_s[idx / GK][idx % GK] = u_r[i];
     }
     __syncthreads();
+    if (k0 + GK < bw) fetch(k0 + GK);
 #pragma unroll 8
     for (int k = 0; k < GK; ++k) {
       const float va = wa_s[ol][k], vi = wi_s[ol][k];
@@ -566,7 +588,7 @@ extern "C" int kvc_rglru_gates(float* a_out, float* drive, const float* u, const
   if (T < 0 || W <= 0 || nb <= 0 || W % nb) return kvc_fail("kvc_rglru_gates: bad sizes");
   if (T == 0) return 0;
   const int bw = W / nb;
-  const bool few = T <= 2 * GT;  // few tokens: smaller tiles of outputs, four times the blocks
+  const bool few = T <= 16 * GT;  // few tokens: smaller tiles of outputs, four times the blocks
   const int go = few ? 16 : 64;
   const int out_tiles = (bw + go - 1) / go;
   const dim3 grid((T + GT - 1) / GT, nb * out_tiles);  // tokens on x, which has no 16-bit limit

@@ -200,3 +200,43 @@ def test_greedy_generation_through_the_engine(models, name, dtype):
             assert int(torch.argmax(row)) == tok, f"{rid}: token {i}"
             checked += 1
     assert checked > 40
+
+
+def test_command_lines(models, tmp_path):
+    """``bin/kvcore_offline_batch`` generates with a Dirulorn folder, and ``bin/trace_run``
+    replays steps on it and writes logits that match the plain model's."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    repo = Path(__file__).resolve().parent.parent
+    folder, cfg, weights, page = models["P"]
+    cmd = [sys.executable, str(repo / "bin" / "kvcore_offline_batch"), "--model", str(folder),
+           "--dtype", "float32", "--prompt-lens", "7,16", "--max-tokens", "5", "--seed", "3",
+           "--max-num-seqs", "4", "--max-num-scheduled-tokens", "32", "--num-gpu-blocks", "32",
+           "--block-size", str(page), "--max-model-len", "128",
+           "--ignore-eos", "--log-level", "WARNING", "--no-log-file"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.count("finish_reason=length") == 2
+
+    tokens = random_tokens(21, cfg["vocab"], 17)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": tokens[:13], "want": [0, 12]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": tokens[13:15], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": tokens[15:], "want": [5]}], "end": ["x"]}]
+    out_dir = tmp_path / "logits"
+    cmd = [str(repo / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out_dir),
+           "--max-tokens", "64", "--block-size", str(page)]
+    proc = subprocess.run(cmd, input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True,
+                          text=True, timeout=240)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not (out_dir / "1.f32").exists()
+    want = oracle("P", cfg, weights, tokens)
+    got = {("x", 0): torch.from_numpy(np.fromfile(out_dir / "0.f32", dtype="<f4").reshape(2, -1)[0]).double(),
+           ("x", 12): torch.from_numpy(np.fromfile(out_dir / "0.f32", dtype="<f4").reshape(2, -1)[1]).double(),
+           ("x", 20): torch.from_numpy(np.fromfile(out_dir / "2.f32", dtype="<f4").reshape(1, -1)[0]).double()}
+    compare(got, {"x": want}, torch.float32)
