@@ -300,10 +300,10 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
     return kvc_fail("kvc_qk_norm_rope_kv_write: one to four value planes that divide the value size");
   if (T == 0) return 0;
   const int v_chunk = dv / num_v_planes;
-  // few tokens: a block per four heads, so that the launch has blocks enough; many tokens: a
-  // block per token walks the heads
+  // a block per token and four heads (up to sixteen such blocks a token, which walk the heads
+  // beyond): blocks enough also for a few tokens, and two barriers a block
   const int all_groups = (nh + nkv + 3) / 4;
-  const int head_groups = T >= 512 ? 1 : (all_groups < 16 ? all_groups : 16);
+  const int head_groups = all_groups < 16 ? all_groups : 16;
   KVC_DISPATCH_DTYPE(
       dtype, Tp, ValuePlanes<Tp> planes{};
       for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);

@@ -61,6 +61,63 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   *o = from_float<TO>(acc);
 }
 
+// The same for up to 8 taps, eight consecutive tokens a thread: the taps' weights are fetched
+// once, and the window of the last K inputs slides along in registers, so that a token costs
+// one load of x and one store.
+constexpr int kConvTokens = 8, kConvMaxTaps = 8;
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void causal_conv_window_kernel(
+    TO* __restrict__ out, int64_t out_stride, const TI* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int T, int C, int K,
+    int act) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int t0 = blockIdx.x * kConvTokens;
+  if (c >= C) return;
+  float wr[kConvMaxTaps], h[kConvMaxTaps];  // wr[j] weighs the input j positions back
+#pragma unroll
+  for (int j = 0; j < kConvMaxTaps; ++j) {
+    wr[j] = j < K ? w[static_cast<int64_t>(c) * K + K - 1 - j] : 0.f;
+    h[j] = 0.f;
+  }
+  const float b0 = bias != nullptr ? bias[c] : 0.f;
+  bool sliding = false;  // h holds the window of the token before
+  for (int tt = 0; tt < kConvTokens && t0 + tt < T; ++tt) {
+    const int t = t0 + tt;
+    TO* o = out + static_cast<int64_t>(t) * out_stride + c;
+    const int r = token_req[t];
+    if (r < 0) {
+      *o = from_float<TO>(0.f);
+      sliding = false;
+      continue;
+    }
+    const int p = positions[t];
+    const int i = t - q_start[r];
+    if (sliding && i > 0) {  // the token before is the same request's, one position back
+#pragma unroll
+      for (int j = kConvMaxTaps - 1; j > 0; --j) h[j] = h[j - 1];
+      h[0] = to_float(x[static_cast<int64_t>(t) * x_stride + c]);
+    } else {
+      const float* st = state + static_cast<int64_t>(slots[r]) * (K - 1) * C + c;
+#pragma unroll
+      for (int j = 0; j < kConvMaxTaps; ++j) {
+        float v = 0.f;
+        if (j < K && j <= p)
+          v = (i - j >= 0) ? to_float(x[static_cast<int64_t>(t - j) * x_stride + c])
+                           : st[static_cast<int64_t>(K - 1 + i - j) * C];
+        h[j] = v;
+      }
+      sliding = true;
+    }
+    float acc = b0;
+#pragma unroll
+    for (int j = 0; j < kConvMaxTaps; ++j) acc = fmaf(wr[j], h[j], acc);
+    if (act == 1) acc = silu_f(acc);
+    *o = from_float<TO>(acc);
+  }
+}
+
 // The state after the step: the last K-1 inputs.  A thread per (request, channel) moves what
 // stays of the old state forward and appends the step's inputs; entry j only reads entries
 // behind it, so rising j works in place.
@@ -568,11 +625,21 @@ extern "C" int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, con
   if (T == 0 || R == 0) return 0;
   const dim3 grid(T, (C + 255) / 256);
   if (grid.y > 65535u) return kvc_fail("kvc_causal_conv: too many channels for one launch");
-  KVC_DISPATCH_2(x_dtype, TI, out_dtype, TO,
-                 hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), grid, dim3(256), 0, S(stream),
-                                    static_cast<TO*>(out), out_stride, static_cast<const TI*>(x),
-                                    x_stride, weight, bias, state, positions, token_req, q_start,
-                                    slots, C, K, act));
+  if (K <= kConvMaxTaps && T >= 4 * kConvTokens) {
+    // many tokens: eight a thread, the window in registers
+    const dim3 tiles((T + kConvTokens - 1) / kConvTokens, (C + 255) / 256);
+    KVC_DISPATCH_2(x_dtype, TI, out_dtype, TO,
+                   hipLaunchKernelGGL((causal_conv_window_kernel<TI, TO>), tiles, dim3(256), 0, S(stream),
+                                      static_cast<TO*>(out), out_stride, static_cast<const TI*>(x),
+                                      x_stride, weight, bias, state, positions, token_req, q_start,
+                                      slots, T, C, K, act));
+  } else {
+    KVC_DISPATCH_2(x_dtype, TI, out_dtype, TO,
+                   hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), grid, dim3(256), 0, S(stream),
+                                      static_cast<TO*>(out), out_stride, static_cast<const TI*>(x),
+                                      x_stride, weight, bias, state, positions, token_req, q_start,
+                                      slots, C, K, act));
+  }
   int rc = kvc_check_launch("kvc_causal_conv");
   if (rc != 0 || !update_state || K == 1) return rc;
   KVC_DISPATCH_DTYPE(x_dtype, TI,

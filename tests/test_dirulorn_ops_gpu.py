@@ -120,12 +120,12 @@ def run_conv_in_steps(ops, x, w, b, cuts, act, slot, state, junk_rows=3):
 @pytest.mark.parametrize("K", [1, 2, 4, 5])
 @pytest.mark.parametrize("act", ["none", "silu"])
 def test_causal_convolution_whole_and_in_steps(ops, K, act):
-    T, C = 23, 70
+    T, C = 53, 70  # steps of 32 tokens and more run the kernel that slides a window along
     x, w, b = rnd(T, C, seed=K), rnd(C, K, seed=K + 10), rnd(C, seed=K + 20)
     want = plain.causal_conv(x.double(), w.double(), b.double())
     if act == "silu":
         want = plain.silu(want)
-    for cuts in ([T], [1] * T, [2, 2, 1, 3, 1, 1, 2, 11], [5, 1, 1, 1, 15], [22, 1]):
+    for cuts in ([T], [1] * T, [2, 2, 1, 3, 1, 1, 2, 11, 30], [5, 1, 1, 1, 15, 30], [52, 1], [1, 52]):
         # a slot that another request has left full of its inputs: the first tokens see zeros
         state = torch.full((3, max(K - 1, 1), C), 7.0, device=DEV)[:, : K - 1]
         got = run_conv_in_steps(ops, x, w, b, cuts, act, slot=1, state=state)
