@@ -625,8 +625,9 @@ extern "C" int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, con
   if (T == 0 || R == 0) return 0;
   const dim3 grid(T, (C + 255) / 256);
   if (grid.y > 65535u) return kvc_fail("kvc_causal_conv: too many channels for one launch");
-  if (K <= kConvMaxTaps && T >= 4 * kConvTokens) {
-    // many tokens: eight a thread, the window in registers
+  if (K <= kConvMaxTaps && T >= 4 * kConvTokens && T >= 4 * static_cast<int64_t>(R)) {
+    // portions of prompts (several tokens a request): eight tokens a thread, the window in
+    // registers; single tokens of many requests would refill the window at every token
     const dim3 tiles((T + kConvTokens - 1) / kConvTokens, (C + 255) / 256);
     KVC_DISPATCH_2(x_dtype, TI, out_dtype, TO,
                    hipLaunchKernelGGL((causal_conv_window_kernel<TI, TO>), tiles, dim3(256), 0, S(stream),
