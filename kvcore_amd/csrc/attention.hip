@@ -213,8 +213,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
   const float* cs = cos_tab + static_cast<int64_t>(t) * half;
   const float* sn = sin_tab + static_cast<int64_t>(t) * half;
 
-  // blockIdx.y deals the heads out four at a time (a wave each); the block with y = 0 also
-  // copies the values
+  // blockIdx.y deals the heads out four at a time (a wave each)
   for (int head_base = 4 * blockIdx.y; head_base < nh + nkv; head_base += 4 * gridDim.y) {
     const bool live = head_base + wave < nh + nkv;
     const int head = live ? head_base + wave : 0;
@@ -267,11 +266,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     }
     __syncthreads();
   }
-  if (!store_kv || blockIdx.y != 0) return;
-  // element i of a value head goes to plane i / v_chunk, V[page, kv head, i % v_chunk, offset]
+  if (!store_kv) return;
+  // element i of a value head goes to plane i / v_chunk, V[page, kv head, i % v_chunk, offset];
+  // the token's blocks share the copy
   const T* vrow = row + static_cast<int64_t>(nh + nkv) * d;
   const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * v_chunk + off;
-  for (int w = threadIdx.x; w < nkv * dv; w += blockDim.x) {
+  for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < nkv * dv; w += blockDim.x * gridDim.y) {
     const int head = w / dv, i = w - head * dv;
     const int c = i / v_chunk, ii = i - c * v_chunk;
     v_planes.plane[c][v_base + (static_cast<int64_t>(head) * v_chunk + ii) * page_size] = vrow[w];

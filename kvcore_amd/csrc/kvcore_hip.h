@@ -158,11 +158,13 @@ int kvc_add_row(float* x, const float* v, int T, int H, kvc_stream stream);
 // act 0 none or 1 silu, in() being zero before the sequence's start; state [slots, K-1, C]
 // float32 holds the K-1 inputs before the step and, with update_state, afterwards those before
 // the next.  x and out are rows of their dtypes with strides (x may be columns of a wider row).
+// single_tokens: the caller vouches that every request brings exactly one token (T = R); the
+// state then moves on in the convolution's own kernel instead of a second one.
 int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                     int x_dtype, const float* weight, const float* bias, float* state,
                     const int32_t* positions, const int32_t* token_req, const int32_t* q_start,
                     const int32_t* slots, int T, int R, int C, int K, int act, int update_state,
-                    kvc_stream stream);
+                    int single_tokens, kvc_stream stream);
 // Gates of the real-gated linear recurrent unit on u [T, W] float32, W in nb blocks: r =
 // sigmoid(wa[b] u_b + ba), i = sigmoid(wi[b] u_b + bi) (wa, wi [nb, W/nb, W/nb] float32, [out,
 // in]); a_out = exp(-c_decay * r * softplus(lam)); drive = sqrt(1 - a^2) * i * u.

@@ -35,9 +35,10 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     TO* __restrict__ out, int64_t out_stride, const TI* __restrict__ x, int64_t x_stride,
-    const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
+    const float* __restrict__ w, const float* __restrict__ bias, float* state,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
-    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int C, int K, int act) {
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int C, int K, int act,
+    int shift_state) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   const int t = blockIdx.x;
   if (c >= C) return;
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   }
   const int p = positions[t];
   const int i = t - q_start[r];
-  const float* st = state + static_cast<int64_t>(slots[r]) * (K - 1) * C + c;
+  float* st = state + static_cast<int64_t>(slots[r]) * (K - 1) * C + c;
   float acc = bias != nullptr ? bias[c] : 0.f;
   const float* wc = w + static_cast<int64_t>(c) * K;
   for (int j = 0; j < K && j <= p; ++j) {
@@ -59,6 +60,12 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   }
   if (act == 1) acc = silu_f(acc);
   *o = from_float<TO>(acc);
+  if (shift_state) {
+    // the token is its request's only one in this step and this thread the only one that
+    // touches the request's state of this channel: the state moves on here, in place
+    for (int j = 0; j + 1 < K - 1; ++j) st[static_cast<int64_t>(j) * C] = st[static_cast<int64_t>(j + 1) * C];
+    if (K > 1) st[static_cast<int64_t>(K - 2) * C] = to_float(x[static_cast<int64_t>(t) * x_stride + c]);
+  }
 }
 
 // The same for up to 8 taps, eight consecutive tokens a thread: the taps' weights are fetched
@@ -618,14 +625,17 @@ extern "C" int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, con
                                int64_t x_stride, int x_dtype, const float* weight, const float* bias,
                                float* state, const int32_t* positions, const int32_t* token_req,
                                const int32_t* q_start, const int32_t* slots, int T, int R, int C,
-                               int K, int act, int update_state, kvc_stream stream) {
+                               int K, int act, int update_state, int single_tokens,
+                               kvc_stream stream) {
   if (T < 0 || R < 0 || C <= 0 || K <= 0 || out_stride < C || x_stride < C)
     return kvc_fail("kvc_causal_conv: bad sizes");
   if (act != 0 && act != 1) return kvc_fail("kvc_causal_conv: activation 0 (none) or 1 (silu)");
   if (T == 0 || R == 0) return 0;
   const dim3 grid(T, (C + 255) / 256);
   if (grid.y > 65535u) return kvc_fail("kvc_causal_conv: too many channels for one launch");
-  if (K <= kConvMaxTaps && T >= 4 * kConvTokens && T >= 4 * static_cast<int64_t>(R)) {
+  // steps of single tokens (the caller says so): the state moves on in the same kernel
+  const int fused = (update_state && single_tokens && T == R) ? 1 : 0;
+  if (!fused && K <= kConvMaxTaps && T >= 4 * kConvTokens && T >= 4 * static_cast<int64_t>(R)) {
     // portions of prompts (several tokens a request): eight tokens a thread, the window in
     // registers; single tokens of many requests would refill the window at every token
     const dim3 tiles((T + kConvTokens - 1) / kConvTokens, (C + 255) / 256);
@@ -639,10 +649,10 @@ extern "C" int kvc_causal_conv(void* out, int64_t out_stride, int out_dtype, con
                    hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), grid, dim3(256), 0, S(stream),
                                       static_cast<TO*>(out), out_stride, static_cast<const TI*>(x),
                                       x_stride, weight, bias, state, positions, token_req, q_start,
-                                      slots, C, K, act));
+                                      slots, C, K, act, fused));
   }
   int rc = kvc_check_launch("kvc_causal_conv");
-  if (rc != 0 || !update_state || K == 1) return rc;
+  if (rc != 0 || !update_state || K == 1 || fused) return rc;
   KVC_DISPATCH_DTYPE(x_dtype, TI,
                      hipLaunchKernelGGL((conv_state_kernel<TI>), dim3(R, (C + 255) / 256), dim3(256),
                                         0, S(stream), state, static_cast<const TI*>(x), x_stride,

@@ -52,7 +52,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_rms_branches_mean": [P, P, P, I, F, I, I, I, P],
         "kvc_concat2": [P, P, P, I, I, I, P],
         "kvc_add_row": [P, P, I, I, P],
-        "kvc_causal_conv": [P, L, I, P, L, I, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "kvc_causal_conv": [P, L, I, P, L, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "kvc_rglru_gates": [P, P, P, P, P, P, P, P, F, I, I, I, P],
         "kvc_rglru_scan": [P, I, P, P, P, L, I, P, P, P, P, P, I, I, I, P, L, P],
         "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
@@ -1077,10 +1077,11 @@ def _rows(t: torch.Tensor, name: str, cols: int) -> tuple[int, int, int]:
 def causal_conv(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
                 state: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
                 q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int, act: str = "none",
-                update_state: bool = True) -> None:
+                update_state: bool = True, single_tokens: bool = False) -> None:
     """Causal convolution per channel over each request's tokens (see the C header): ``x [T, C]``
     (a column view is fine), ``weight [C, K]`` float32 with the last column the current token's,
-    ``state [slots, K-1, C]`` float32 (read, and with ``update_state`` rewritten)."""
+    ``state [slots, K-1, C]`` float32 (read, and with ``update_state`` rewritten).
+    ``single_tokens``: every request brings exactly one token, which lets one kernel do both."""
     T, C = x.shape
     K = weight.shape[1]
     if weight.shape != (C, K) or (bias is not None and bias.shape != (C,)):
@@ -1096,7 +1097,7 @@ def causal_conv(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: 
         None if bias is None else _dev(bias, "bias", torch.float32), _dev(state, "state"),
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs, C, K,
-        {"none": 0, "silu": 1}[act], int(update_state), _stream()), "kvc_causal_conv")
+        {"none": 0, "silu": 1}[act], int(update_state), int(bool(single_tokens)), _stream()), "kvc_causal_conv")
 
 
 def rglru_gates(a_out: torch.Tensor, drive: torch.Tensor, u: torch.Tensor, wa: torch.Tensor,

@@ -95,7 +95,8 @@ class GatedLinearRecurrence(Mixer):
         yx = ctx.buf(f"lru_yx:{2 * W}", 2 * W)
         ops.linear(yx, x, p["yx.weight"], p["yx.bias"])
         u = ctx.buf(f"lru_u:{W}", W, torch.float32)
-        ops.causal_conv(u, yx[:, W:], p["conv.weight"], p["conv.bias"], conv_state, act="none", **batch)
+        ops.causal_conv(u, yx[:, W:], p["conv.weight"], p["conv.bias"], conv_state, act="none",
+                        single_tokens=ctx.max_query_len == 1, **batch)
         a = ctx.buf(f"lru_a:{W}", W, torch.float32)
         drive = ctx.buf(f"lru_drive:{W}", W, torch.float32)
         ops.rglru_gates(a, drive, u, p["gate_a.weight"], p["gate_i.weight"], p["gate_a.bias"],
@@ -187,7 +188,8 @@ class StateSpaceMixer(Mixer):
         xbc_raw = proj[:, self.inner: self.inner + self.conv_dim]
         dt_raw = proj[:, self.inner + self.conv_dim:]
         xbc = ctx.buf(f"ssm_xbc:{self.conv_dim}", self.conv_dim, torch.float32)
-        ops.causal_conv(xbc, xbc_raw, p["conv.weight"], p["conv.bias"], conv_state, act="silu", **batch)
+        ops.causal_conv(xbc, xbc_raw, p["conv.weight"], p["conv.bias"], conv_state, act="silu",
+                        single_tokens=ctx.max_query_len == 1, **batch)
         y = ctx.buf(f"ssm_y:{self.inner}", self.inner, torch.float32)
         ops.ssm_scan(y, xbc, dt_raw, p["dt_bias"], p["A_log"], p["D"], ssm_state, heads=self.heads,
                      head_dim=self.head_dim, state_size=self.state_size, groups=self.groups, **batch)

@@ -132,6 +132,33 @@ def test_causal_convolution_whole_and_in_steps(ops, K, act):
         close(got, want, 1e-5)
 
 
+@pytest.mark.parametrize("K", [1, 2, 4])
+def test_convolution_of_single_tokens_moves_its_state_on_in_the_same_kernel(ops, K):
+    """A step in which every request brings one token (as the caller vouches): two requests at
+    different positions and a padded row between them, token after token."""
+    T, C = 19, 40
+    xa, xb = rnd(T, C, seed=1), rnd(T, C, seed=2)
+    w, b = rnd(C, K, seed=3), rnd(C, seed=4)
+    want_a = plain.causal_conv(xa.double(), w.double(), b.double())
+    want_b = plain.causal_conv(xb.double(), w.double(), b.double())
+    state = torch.full((3, max(K - 1, 1), C), 5.0, device=DEV)[:, : K - 1]
+    got_a, got_b = [], []
+    for t in range(T):
+        reqs = [(2, t, 1), None] + ([(0, t - 4, 1)] if t >= 4 else [])  # the second starts four steps later
+        batch, total = batch_tensors(reqs)
+        rows = torch.zeros(total, C)
+        rows[0] = xa[t]
+        if t >= 4:
+            rows[2] = xb[t - 4]
+        out = torch.full((total, C), float("nan"), device=DEV)
+        ops.causal_conv(out, rows.to(DEV), w.to(DEV), b.to(DEV), state, single_tokens=True, **batch)
+        got_a.append(out[0].cpu())
+        if t >= 4:
+            got_b.append(out[2].cpu())
+    close(torch.stack(got_a), want_a, 1e-5)
+    close(torch.stack(got_b), want_b[: T - 4], 1e-5)
+
+
 def test_convolution_reads_bfloat16_rows_and_writes_them(ops):
     T, C, K = 9, 32, 4
     x, w = rnd(T, C, seed=1, dtype=torch.bfloat16), rnd(C, K, seed=2)
