@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
     int interleaved, const int32_t* __restrict__ kv_slot, int nh, int nkv, int d, int dv,
-    int page_size, int write_kv) {
+    int page_size, int write_kv, int copy_values) {
   __shared__ float head_s[4][kMaxHeadDim];
   const int t = blockIdx.x;
   const int slot = kv_slot[t];
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     }
     __syncthreads();
   }
-  if (!store_kv) return;
+  if (!store_kv || !copy_values) return;
   // element i of a value head goes to plane i / v_chunk, V[page, kv head, i % v_chunk, offset];
   // the token's blocks share the copy
   const T* vrow = row + static_cast<int64_t>(nh + nkv) * d;
@@ -275,6 +275,101 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     const int head = w / dv, i = w - head * dv;
     const int c = i / v_chunk, ii = i - c * v_chunk;
     v_planes.plane[c][v_base + (static_cast<int64_t>(head) * v_chunk + ii) * page_size] = vrow[w];
+  }
+}
+
+// The same norm, rotation and key write for heads of up to 64 elements: a wave per (token,
+// head) with an element a lane; a rotary pair's partner is a lane away (its neighbour, or half
+// the rotated width apart), so the wave needs neither LDS nor a barrier.  The values are left
+// to the kernel below.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_k_write_small_kernel(
+    T* __restrict__ qkv, int64_t row_stride, T* __restrict__ k_cache,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
+    int interleaved, const int32_t* __restrict__ kv_slot, int num_tokens, int nh, int nkv, int d,
+    int page_size, int write_kv) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  const int heads = nh + nkv;
+  if (item >= static_cast<int64_t>(num_tokens) * heads) return;  // the whole wave
+  const int t = static_cast<int>(item / heads);
+  const int head = static_cast<int>(item - static_cast<int64_t>(t) * heads);
+  const int slot = kv_slot[t];
+  if (slot == -2) return;  // padding token
+  const int half = rot_dim / 2;
+  T* hp = qkv + static_cast<int64_t>(t) * row_stride + static_cast<int64_t>(head) * d;
+  const bool in = lane < d;
+  float x = in ? to_float(hp[lane]) : 0.f;
+  const float* gain = head < nh ? q_gain : k_gain;
+  if (gain != nullptr) {
+    const float ss = wave_sum(x * x);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(d) + eps);
+    if (in) x = x * inv * gain[lane];
+  }
+  // the pair's other element, from its lane (every lane takes part in the exchange)
+  int partner, j;
+  bool first;
+  if (interleaved) {
+    partner = lane ^ 1; j = lane >> 1; first = (lane & 1) == 0;
+  } else {
+    first = lane < half; j = first ? lane : lane - half; partner = first ? lane + half : lane - half;
+  }
+  const float other = __shfl(x, partner & (kWave - 1), kWave);
+  float y = x;
+  if (lane < rot_dim) {
+    const float c = cos_tab[static_cast<int64_t>(t) * half + j], sn = sin_tab[static_cast<int64_t>(t) * half + j];
+    y = first ? rotate_first(x, other, c, sn) : rotate_second(other, x, c, sn);
+  }
+  if (!in) return;
+  const T r = from_float<T>(y);
+  hp[lane] = r;
+  if (head >= nh && write_kv && slot >= 0) {
+    const int page = slot / page_size, off = slot - page * page_size;
+    k_cache[((static_cast<int64_t>(page) * nkv + (head - nh)) * page_size + off) * d + lane] = r;
+  }
+}
+
+// The values of eight consecutive tokens a block, for steps of many tokens.  A V page keeps the
+// keys side by side, so a token alone stores its values two or four bytes at a time, page_size
+// elements apart; when the block's eight tokens lie side by side in one page (a portion of a
+// prompt mostly does), a thread gathers one element of all eight and stores them together.
+template <typename T>
+__global__ __launch_bounds__(256) void value_planes_write_tile_kernel(
+    const T* __restrict__ qkv, int64_t row_stride, ValuePlanes<T> v_planes, int v_chunk,
+    const int32_t* __restrict__ kv_slot, int num_tokens, int v_begin, int nkv, int dv, int page_size) {
+  constexpr int TILE = 8;
+  const int t0 = blockIdx.x * TILE;
+  const int n_tok = (num_tokens - t0 < TILE) ? num_tokens - t0 : TILE;
+  const int s0 = kv_slot[t0];
+  bool side_by_side = n_tok == TILE && s0 >= 0 && (s0 & 7) == 0 && (page_size & 7) == 0;
+  for (int ti = 1; ti < n_tok; ++ti) side_by_side = side_by_side && kv_slot[t0 + ti] == s0 + ti;
+  if (side_by_side) {
+    const int page = s0 / page_size, off = s0 - page * page_size;
+    const int64_t v_base = static_cast<int64_t>(page) * nkv * page_size * v_chunk + off;
+    for (int w = threadIdx.x; w < nkv * dv; w += blockDim.x) {
+      const int head = w / dv, i = w - head * dv;
+      const int c = i / v_chunk, ii = i - c * v_chunk;
+      const T* src = qkv + static_cast<int64_t>(t0) * row_stride + v_begin + w;
+      alignas(16) T vals[TILE];
+#pragma unroll
+      for (int ti = 0; ti < TILE; ++ti) vals[ti] = src[ti * row_stride];
+      T* dst = v_planes.plane[c] + v_base + (static_cast<int64_t>(head) * v_chunk + ii) * page_size;
+      *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(vals);
+      if constexpr (sizeof(T) == 4) *reinterpret_cast<uint4*>(dst + 4) = *reinterpret_cast<const uint4*>(vals + 4);
+    }
+    return;
+  }
+  for (int w = threadIdx.x; w < n_tok * nkv * dv; w += blockDim.x) {
+    const int ti = w / (nkv * dv), rest = w - ti * nkv * dv;
+    const int slot = kv_slot[t0 + ti];
+    if (slot < 0) continue;
+    const int page = slot / page_size, off = slot - page * page_size;
+    const int head = rest / dv, i = rest - head * dv;
+    const int c = i / v_chunk, ii = i - c * v_chunk;
+    v_planes.plane[c][static_cast<int64_t>(page) * nkv * page_size * v_chunk + off +
+                      (static_cast<int64_t>(head) * v_chunk + ii) * page_size] =
+        qkv[static_cast<int64_t>(t0 + ti) * row_stride + v_begin + rest];
   }
 }
 
@@ -304,6 +399,26 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
   // beyond): blocks enough also for a few tokens, and two barriers a block
   const int all_groups = (nh + nkv + 3) / 4;
   const int head_groups = all_groups < 16 ? all_groups : 16;
+  // steps of many tokens store the values eight tokens at a time, 16 bytes a store (the planes
+  // must be 16-byte aligned for that, which whole pages of 8 tokens and more are)
+  bool tiled_values = write_kv && T >= 16 && page_size % 8 == 0;
+  for (int c = 0; c < num_v_planes; ++c)
+    tiled_values = tiled_values && (reinterpret_cast<uintptr_t>(host_v_planes[c]) & 15) == 0;
+  if (tiled_values && d <= kWave) {
+    // many tokens and heads of up to 64 elements: a wave a head, then the values
+    const int64_t waves = static_cast<int64_t>(T) * (nh + nkv);
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp, ValuePlanes<Tp> planes{};
+        for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
+        hipLaunchKernelGGL(qk_norm_rope_k_write_small_kernel<Tp>, dim3(static_cast<unsigned>((waves + 3) / 4)),
+                           dim3(256), 0, reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv),
+                           row_stride, static_cast<Tp*>(k_cache), q_gain, k_gain, eps, cos_tab, sin_tab,
+                           rot_dim, interleaved, kv_slot, T, nh, nkv, d, page_size, write_kv);
+        hipLaunchKernelGGL(value_planes_write_tile_kernel<Tp>, dim3((T + 7) / 8), dim3(256), 0,
+                           reinterpret_cast<hipStream_t>(stream), static_cast<const Tp*>(qkv), row_stride,
+                           planes, v_chunk, kv_slot, T, (nh + nkv) * d, nkv, dv, page_size));
+    return kvc_check_launch("kvc_qk_norm_rope_kv_write");
+  }
   KVC_DISPATCH_DTYPE(
       dtype, Tp, ValuePlanes<Tp> planes{};
       for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
@@ -311,6 +426,10 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
                          static_cast<Tp*>(k_cache), planes, v_chunk, q_gain, k_gain, eps,
                          cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,
-                         write_kv));
+                         write_kv, tiled_values ? 0 : 1);
+      if (tiled_values) hipLaunchKernelGGL(
+          value_planes_write_tile_kernel<Tp>, dim3((T + 7) / 8), dim3(256), 0,
+          reinterpret_cast<hipStream_t>(stream), static_cast<const Tp*>(qkv), row_stride, planes,
+          v_chunk, kv_slot, T, (nh + nkv) * d, nkv, dv, page_size));
   return kvc_check_launch("kvc_qk_norm_rope_kv_write");
 }

@@ -474,3 +474,44 @@ def test_rotation_pairs_neighbours_and_leaves_the_rest(ops):
         page_id, off = 1 + t // page, t % page
         assert torch.equal(kc[page_id, 0, off].cpu(), rows[t, d: 2 * d])
         assert torch.equal(vc[page_id, 0, :, off].cpu(), qkv[t, 2 * d:])
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("T", [5, 40])  # few tokens: a block a token; many: a wave a head and tiled values
+def test_head_norm_and_rotation_in_both_pairings(ops, interleaved, T):
+    """The rewritten q and k rows and the cache after the kernel, against the norm and rotation
+    written out here: pairs of neighbours, or pairs half the rotated width apart."""
+    nh, nkv, d, dv, rot, page = 3, 2, 32, 16, 16, 8
+    qkv = rnd(T, (nh + nkv) * d + nkv * dv, seed=T)
+    gq, gk = rnd(d, seed=1) * 0.3 + 1, rnd(d, seed=2) * 0.3 + 1
+    freqs = torch.tensor([0.7 ** i for i in range(rot // 2)], dtype=torch.float64)
+    heads = qkv[:, : (nh + nkv) * d].double().view(T, nh + nkv, d)
+    gains = torch.cat([gq.double().expand(nh, d), gk.double().expand(nkv, d)])
+    normed = plain.rms_unit(heads, 1e-5) * gains
+    ang = torch.arange(T, dtype=torch.float64)[:, None] * freqs
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    want = normed.clone()
+    if interleaved:
+        u, v = normed[..., 0:rot:2], normed[..., 1:rot:2]
+        want[..., 0:rot:2], want[..., 1:rot:2] = u * c - v * s, v * c + u * s
+    else:
+        u, v = normed[..., : rot // 2], normed[..., rot // 2: rot]
+        want[..., : rot // 2], want[..., rot // 2: rot] = u * c - v * s, v * c + u * s
+    kc, vc = attention_setup(ops, T + 16, nkv, d, dv, page, torch.float32)
+    table = torch.tensor([[4, 2, 7, 1, 3, 5, 6]], dtype=torch.int32, device=DEV)
+    batch, total = batch_tensors([(0, 0, T)])
+    cos, sin = torch.empty(T, rot // 2, device=DEV), torch.empty(T, rot // 2, device=DEV)
+    ops.rope_table(cos, sin, batch["positions"], freqs.float().to(DEV))
+    kv_slot = torch.empty(T, dtype=torch.int32, device=DEV)
+    ops.kv_slots(kv_slot, positions=batch["positions"], token_req=batch["token_req"], slots=batch["slots"],
+                 table=table, page_size=page, num_pages=kc.shape[0])
+    rows = qkv.to(DEV)
+    ops.qk_norm_rope_kv_write(rows, kc, vc, cos, sin, rot_dim=rot, interleaved=interleaved, kv_slot=kv_slot,
+                              nh=nh, nkv=nkv, d=d, dv=dv, q_gain=gq.to(DEV), k_gain=gk.to(DEV), eps=1e-5)
+    close(rows[:, : (nh + nkv) * d].view(T, nh + nkv, d), want, 2e-5, 1e-5)
+    assert torch.equal(rows[:, (nh + nkv) * d:].cpu(), qkv[:, (nh + nkv) * d:])
+    pages = table[0].tolist()
+    for t in range(T):
+        pg, off = pages[t // page], t % page
+        close(kc[pg, :, off], want[t, nh:], 2e-5, 1e-5)
+        assert torch.equal(vc[pg, :, :, off].cpu(), qkv[t, (nh + nkv) * d:].view(nkv, dv))
