@@ -83,7 +83,16 @@ CONFIG_S = {
     "loop": {"start": 1, "stop": 2, "times": 2},
 }
 
-CONFIGS = {"P": (CONFIG_P, 8), "Q": (CONFIG_Q, 16), "R": (CONFIG_R, 4), "S": (CONFIG_S, 16)}
+# state-space layers only: a model that keeps no paged cache at all, only states
+CONFIG_M = {
+    "architecture": "Dirulorn", "vocab": 150, "width": 48, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "mamba2", "mlp": {"kind": "dense", "ff": 64}, "mixer": _ssm(2, 16, 8, 1, 3, 1)},
+        {"type": "mamba2", "mlp": {"kind": "dense", "ff": 80}, "mixer": _ssm(4, 24, 32, 2, 4, 2)},
+    ],
+}
+
+CONFIGS = {"P": (CONFIG_P, 8), "Q": (CONFIG_Q, 16), "R": (CONFIG_R, 4), "S": (CONFIG_S, 16), "M": (CONFIG_M, 16)}
 
 
 def make_model_dir(folder: Path, config: dict, seed: int) -> Path:

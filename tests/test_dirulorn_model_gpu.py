@@ -162,7 +162,7 @@ def test_attention_runs_on_the_matrix_cores_where_keys_and_values_are_alike(mode
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16"])
-@pytest.mark.parametrize("name", ["P", "Q"])
+@pytest.mark.parametrize("name", ["P", "Q", "M"])
 def test_greedy_generation_through_the_engine(models, name, dtype):
     """``LLMEngine.generate`` with the scheduler cutting prompts into portions of 16 tokens:
     every generated token is the plain model's greedy choice given the tokens before it (a
