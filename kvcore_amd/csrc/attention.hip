@@ -8,7 +8,9 @@
 // accumulators), then the lanes split the head's elements to add p_j * V_j in key
 // order.  K pages are [kv head, page_size, d], V pages [kv head, dv, page_size]: keys of d
 // elements and values of dv, which need not be equal.  What a token computes depends on its position, window and cache content
-// only: not on the batch it is in nor on how its request was cut into steps.
+// only: not on the batch it is in nor on how its request was cut into steps.  Two options:
+// `slopes` (a value per query head) takes slope * (position - key position) off every score, and
+// `chunk` lets a token see only the keys of its own chunk of that many positions.
 
 #include <hip/hip_runtime.h>
 
@@ -46,7 +48,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     const T* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ slots, int nh, int nkv, int d, int dv, int page_size, int num_pages,
-    float scale, int window) {
+    float scale, int window, const float* __restrict__ slopes, int chunk) {
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
   __shared__ float p_s[kWavesPerBlock][kWave];
   __shared__ int64_t off_s[kWavesPerBlock][kWave];   // K row of each key of the tile
@@ -67,9 +69,12 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     return;
   }
   const int pos = positions[t];
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  // chunks are counted from the sequence's first position: a token sees its own chunk's keys
+  if (chunk > 0 && (pos / chunk) * chunk > first) first = (pos / chunk) * chunk;
   const int32_t* row = table + static_cast<int64_t>(slots[req]) * table_stride;
   const int hk = h / (nh / nkv);
+  const float slope = slopes != nullptr ? slopes[h] : 0.f;  // taken off the score per token of distance
 
   const T* qh = q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * d;
   for (int i = lane; i < d; i += kWave) q_s[wave][i] = to_float(qh[i]);
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
         } else {  // a key size that 16-byte loads do not divide: element by element
           for (int i = 0; i < d; ++i) dot = fmaf(q_s[wave][i], to_float(kr[i]), dot);
         }
-        s = dot * scale;
+        s = dot * scale - slope * static_cast<float>(pos - key);
       }
     }
     const float tile_max = wave_max(s);
@@ -155,7 +160,7 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                                    const int32_t* positions, const int32_t* token_req,
                                    const int32_t* slots, int T, int nh, int nkv, int d, int dv,
                                    int page_size, int num_pages, float scale, int window,
-                                   int dtype, kvc_stream stream) {
+                                   const float* slopes, int chunk, int dtype, kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || page_size <= 0 || num_pages <= 0 || table_stride <= 0)
     return kvc_fail("kvc_paged_attention: bad sizes");
   if (nh % nkv) return kvc_fail("kvc_paged_attention: heads must be a multiple of kv heads");
@@ -173,7 +178,8 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(out),
                          static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                          static_cast<const Tp*>(v_cache), table, table_stride, positions,
-                         token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window));
+                         token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window, slopes,
+                         chunk));
   return kvc_check_launch("kvc_paged_attention");
 }
 

@@ -419,6 +419,27 @@ extern "C" int kvc_residual_add(float* residual, const void* delta, int T, int H
 }
 
 // ------------------------------------------------------------------------- SiLU-mul
+template <typename TA, typename TB>
+__global__ void residual_add2_kernel(float* __restrict__ residual, const TA* __restrict__ a,
+                                     const TB* __restrict__ b, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) residual[i] += to_float(a[i]) + to_float(b[i]);
+}
+
+extern "C" int kvc_residual_add2(float* residual, const void* a, int a_dtype, const void* b, int b_dtype,
+                                 int T, int H, kvc_stream stream) {
+  if (T < 0 || H <= 0) return kvc_fail("kvc_residual_add2: bad sizes");
+  const int64_t n = static_cast<int64_t>(T) * H;
+  if (n == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  KVC_DISPATCH_DTYPE(a_dtype, TA,
+                     KVC_DISPATCH_DTYPE(b_dtype, TB,
+                                        hipLaunchKernelGGL((residual_add2_kernel<TA, TB>), dim3(blocks), dim3(256), 0,
+                                                           S(stream), residual, static_cast<const TA*>(a),
+                                                           static_cast<const TB*>(b), n)));
+  return kvc_check_launch("kvc_residual_add2");
+}
+
 template <typename T>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int I,
                                 int64_t n) {

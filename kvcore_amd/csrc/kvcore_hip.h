@@ -76,6 +76,9 @@ int kvc_rmsnorm(void* out, const void* x, const float* weight, float eps, int T,
 // residual += delta, nothing else.
 int kvc_residual_add(float* residual, const void* delta, int T, int H, int dtype,
                      kvc_stream stream);
+// residual[t] += a[t] + b[t] (the two added first), a and b of their own dtypes.
+int kvc_residual_add2(float* residual, const void* a, int a_dtype, const void* b, int b_dtype, int T,
+                      int H, kvc_stream stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i].
 int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype, kvc_stream stream);
@@ -114,11 +117,14 @@ int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_
 // max(0, p - window + 1) .. p (window <= 0: all), read through the block table.
 // q is [T, nh, d] with q_stride elements between tokens; keys have d elements, values dv (K
 // pages [kv head, page_size, d], V pages [kv head, dv, page_size]); out is [T, nh*dv].
+// slopes (float32 [nh], or null): slopes[h] * (p - key position) is taken off every score of head
+// h.  chunk > 0: a token sees only the keys j with j / chunk == p / chunk.
 int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                         const void* v_cache, const int32_t* table, int table_stride,
                         const int32_t* positions, const int32_t* token_req,
                         const int32_t* slots, int T, int nh, int nkv, int d, int dv, int page_size,
-                        int num_pages, float scale, int window, int dtype, kvc_stream stream);
+                        int num_pages, float scale, int window, const float* slopes, int chunk,
+                        int dtype, kvc_stream stream);
 
 // What kvc_rope_kv_write does, for heads whose keys (d) and values (dv) may differ in size,
 // with a norm of every q and k head before the rotation: rows of qkv are [nh q heads of d |
@@ -199,6 +205,58 @@ int kvc_ssm_scan(float* y, const float* xbc, int64_t xbc_stride, const void* dt_
 int kvc_gated_group_rmsnorm(void* out, int out_dtype, const float* y, const void* z,
                             int64_t z_stride, int z_dtype, const float* gain, float eps, int T,
                             int width, int groups, kvc_stream stream);
+
+// ---- mixers whose state is a float32 matrix S [d, dv] per head (linear_attention.hip).  The batch
+// is described as for the recurrent mixers above; state is [slots, nh, d, dv] float32.
+// Per head h (its q and k come from head h / (nh / nqk) of nqk heads of d), token by token:
+//   delta_rule 0:  S = diag(decay[t, h, :]) S + k v^T            (decay rows of nh * d values)
+//   delta_rule 1:  S = decay[t, h] S;  u = beta[t, h] (v - S^T k);  S = S + k u^T
+// and out[t, h] = S^T (q_scale q) after the token's write; out is [T, nh * dv] float32.  q, k, v, decay and
+// beta are float32 rows with strides.  d at most 256.
+int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
+                          int64_t k_stride, const float* v, int64_t v_stride, const float* decay,
+                          int64_t decay_stride, const float* beta, int64_t beta_stride, float* state,
+                          const int32_t* positions, const int32_t* token_req, const int32_t* q_start,
+                          const int32_t* slots, int R, int nh, int nqk, int d, int dv, int delta_rule,
+                          float q_scale, kvc_stream stream);
+// a[t, i] = sigmoid(z[t, i] + bias[i]) ^ inv_tau, computed as exp(inv_tau * log sigmoid); bias may be null.
+int kvc_sigmoid_power(float* a, const float* z, int64_t z_stride, const float* bias, float inv_tau,
+                      int T, int W, kvc_stream stream);
+// g[t, h] = exp(-exp(a_log[h]) * softplus(a_raw[t, h] + dt_bias[h])); beta[t, h] = sigmoid(b_raw[t, h]).
+int kvc_decay_and_write_gates(float* g, float* beta, const float* a_raw, int64_t a_stride,
+                              const float* b_raw, int64_t b_stride, const float* a_log,
+                              const float* dt_bias, int T, int nh, kvc_stream stream);
+// x[t, h, :] *= scale / sqrt(sum x[t, h, :]^2 + eps), in place, heads of d float32 values.
+int kvc_unit_heads(float* x, int64_t stride, int T, int heads, int d, float eps, float scale,
+                   kvc_stream stream);
+// out[t, h, c] = o[t, h, c] / sqrt(mean_c o[t, h, :]^2 + eps) * gain[c] * silu(gate[t, h, c]).
+int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* gate,
+                          int64_t gate_stride, int gate_dtype, const float* gain, float eps, int T,
+                          int heads, int dv, kvc_stream stream);
+
+// ---- routed experts (moe.hip); see the head of that file.  choice and weight are [T, top];
+// sorted [pairs]; tiles [max_tiles, 3] (expert, first sorted row, rows); num_tiles [1].
+// kvc_moe_gemm multiplies every tile's rows by its expert's matrix: w is [E, N, K], or with
+// `gated` [E, 2N, K] (gate rows, then up rows) and the activation applied; a sorted row i reads
+// x row sorted[i] / in_div (in_div 0: row i itself) and writes out row i (out_sorted) or
+// sorted[i].  dtype is that of x and w.
+int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
+                  int groups, int keep, kvc_stream stream);
+int kvc_moe_max_tiles(int pairs, int E);
+int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int32_t* choice,
+                  int pairs, int E, int max_tiles, kvc_stream stream);
+int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
+                 const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
+                 const int32_t* num_tiles, int max_tiles, int N, int K, int in_div, int out_sorted,
+                 int gated, float limit, float alpha, kvc_stream stream);
+// out[t] = sum_c weight[t, c] * y[t * top + c] + add0[t] + add1[t] (either may be null; add0 of
+// dtype add0_dtype, add1 float32), float32.
+int kvc_moe_combine(float* out, const float* y, const float* weight, int top, const void* add0,
+                    int add0_dtype, const float* add1, int T, int H, kvc_stream stream);
+// out[t, i] = g * sigmoid(alpha * g) * (u + 1), g = min(gate_up[t, i], limit),
+// u = clamp(gate_up[t, I + i], -limit, limit).
+int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, float limit, float alpha, int dtype,
+                    kvc_stream stream);
 
 // The same attention for bfloat16 steps of single tokens on the matrix cores, a block of
 // several waves per (token, kv head, split), which also does what kvc_rope_kv_write does for

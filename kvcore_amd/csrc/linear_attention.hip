@@ -1,0 +1,313 @@
+// Mixers whose memory is a matrix per head, S [d, dv] in float32, carried from token to token
+// (linear attention and its kin), and the small float32 kernels around them.
+//
+// kvc_linear_state_scan walks each request's tokens in order.  Two update rules:
+//   key decay   S <- diag(a_t) S + k_t v_t^T                      (a_t one factor per key channel)
+//   delta rule  S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T   (g_t, beta_t scalars)
+// and in both o_t = S^T (q_scale q_t), read after the token's write.  A block owns one (request, head, tile
+// of VT value channels); the NSL threads that share a column of the state are neighbouring lanes
+// (their partial sums meet through lane shuffles, in one fixed order) and each keeps NPT rows in
+// registers; q, k, the factors and v of 16 tokens at a time go through LDS.  A request whose
+// first token of the step is at position 0 starts from zero, any other from its slot's state;
+// the state goes back to the slot at the end.  What a token's result is depends on its request's
+// earlier tokens only, not on how they were cut into steps or what else the batch holds.
+
+#include <hip/hip_runtime.h>
+
+#include "device_utils.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+namespace {
+
+#define S(stream) reinterpret_cast<hipStream_t>(stream)
+
+constexpr int LSC = 16;  // tokens a stage
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float silu_ff(float x) { return x / (1.f + expf(-x)); }
+// log(1 + e^x) without a threshold: max(x, 0) + log1p(e^-|x|)
+__device__ __forceinline__ float softplus_ff(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+// log(sigmoid(x)) = -softplus(-x)
+__device__ __forceinline__ float log_sigmoid_f(float x) { return -softplus_ff(-x); }
+
+template <int NPT, int DELTA>
+__global__ __launch_bounds__(256) void linear_state_scan_kernel(
+    float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
+    int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ decay,
+    int64_t decay_stride, const float* __restrict__ beta, int64_t beta_stride, float* __restrict__ state,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int nqk, int d,
+    int dv, int VT, int NSL, float q_scale) {
+  extern __shared__ float lds[];
+  float* q_s = lds;               // [LSC][d]
+  float* k_s = q_s + LSC * d;     // [LSC][d]
+  float* a_s = k_s + LSC * d;     // [LSC][d] (key decay) or [LSC][2] (delta: g, beta)
+  float* v_s = a_s + LSC * (DELTA ? 2 : d);  // [LSC][VT]
+  const int r = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * VT;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int ns = tid % NSL, pl = tid / NSL;
+  const int c = c0 + pl;
+  const bool c_ok = c < dv;
+  const int width = nh * dv;
+  const int b = q_start[r], e = q_start[r + 1];
+  if (e <= b) return;
+  if (token_req[b] < 0) {  // padding rows: zeros out, no state touched
+    for (int idx = tid; idx < (e - b) * VT; idx += nthreads) {
+      const int tt = idx / VT, cc = c0 + idx - tt * VT;
+      if (cc < dv) out[static_cast<int64_t>(b + tt) * width + h * dv + cc] = 0.f;
+    }
+    return;
+  }
+  const int hk = h / (nh / nqk);
+  float* st = state + (static_cast<int64_t>(slots[r]) * nh + h) * d * dv;
+  const bool fresh = positions[b] == 0;
+  float s[NPT];
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) {
+    const int n = ns + NSL * i;
+    s[i] = (!fresh && c_ok && n < d) ? st[static_cast<int64_t>(n) * dv + c] : 0.f;
+  }
+  for (int t0 = b; t0 < e; t0 += LSC) {
+    const int nt = (e - t0 < LSC) ? e - t0 : LSC;
+    __syncthreads();
+    for (int idx = tid; idx < nt * d; idx += nthreads) {
+      const int tt = idx / d, n = idx - tt * d;
+      const int64_t t = t0 + tt;
+      q_s[idx] = q[t * q_stride + hk * d + n] * q_scale;
+      k_s[idx] = k[t * k_stride + hk * d + n];
+      if (!DELTA) a_s[idx] = decay[t * decay_stride + h * d + n];
+    }
+    if (DELTA) {
+      for (int tt = tid; tt < nt; tt += nthreads) {
+        a_s[2 * tt] = decay[static_cast<int64_t>(t0 + tt) * decay_stride + h];
+        a_s[2 * tt + 1] = beta[static_cast<int64_t>(t0 + tt) * beta_stride + h];
+      }
+    }
+    for (int idx = tid; idx < nt * VT; idx += nthreads) {
+      const int tt = idx / VT, cc = c0 + idx - tt * VT;
+      v_s[idx] = cc < dv ? v[static_cast<int64_t>(t0 + tt) * v_stride + h * dv + cc] : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* qt = q_s + tt * d;
+      const float* kt = k_s + tt * d;
+      const float vv = v_s[tt * VT + pl];
+      float acc = 0.f;
+      if (DELTA) {
+        const float g = a_s[2 * tt], bt = a_s[2 * tt + 1];
+        float kd = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+          const int n = ns + NSL * i;
+          if (n < d) {
+            s[i] *= g;
+            kd = fmaf(s[i], kt[n], kd);
+          }
+        }
+        for (int o = 1; o < NSL; o <<= 1) kd += __shfl_xor(kd, o, kWave);
+        const float u = bt * (vv - kd);
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+          const int n = ns + NSL * i;
+          if (n < d) {
+            s[i] = fmaf(kt[n], u, s[i]);
+            acc = fmaf(s[i], qt[n], acc);
+          }
+        }
+      } else {
+        const float* at = a_s + tt * d;
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+          const int n = ns + NSL * i;
+          if (n < d) {
+            s[i] = fmaf(at[n], s[i], kt[n] * vv);
+            acc = fmaf(s[i], qt[n], acc);
+          }
+        }
+      }
+      for (int o = 1; o < NSL; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+      if (ns == 0 && c_ok) out[static_cast<int64_t>(t0 + tt) * width + h * dv + c] = acc;
+    }
+  }
+  if (!c_ok) return;
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) {
+    const int n = ns + NSL * i;
+    if (n < d) st[static_cast<int64_t>(n) * dv + c] = s[i];
+  }
+}
+
+// a[t, i] = exp(log(sigmoid(z[t, i] + bias[i])) * inv_tau): sigmoid(z)^(1/tau), through its logarithm
+__global__ __launch_bounds__(256) void sigmoid_power_kernel(float* __restrict__ a, const float* __restrict__ z,
+                                                             int64_t z_stride, const float* __restrict__ bias,
+                                                             float inv_tau, int T, int W) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<int64_t>(T) * W) return;
+  const int t = static_cast<int>(idx / W), i = static_cast<int>(idx - static_cast<int64_t>(t) * W);
+  const float x = z[t * z_stride + i] + (bias != nullptr ? bias[i] : 0.f);
+  a[idx] = expf(log_sigmoid_f(x) * inv_tau);
+}
+
+// g[t, h] = exp(-exp(a_log[h]) * softplus(a_raw[t, h] + dt_bias[h])); beta[t, h] = sigmoid(b_raw[t, h])
+__global__ __launch_bounds__(256) void decay_and_write_gates_kernel(
+    float* __restrict__ g, float* __restrict__ beta, const float* __restrict__ a_raw, int64_t a_stride,
+    const float* __restrict__ b_raw, int64_t b_stride, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, int T, int nh) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * nh) return;
+  const int t = idx / nh, h = idx - t * nh;
+  g[idx] = expf(-expf(a_log[h]) * softplus_ff(a_raw[t * a_stride + h] + dt_bias[h]));
+  beta[idx] = sigmoid_f(b_raw[t * b_stride + h]);
+}
+
+// Heads of d float32 values made unit vectors in place, x / sqrt(sum x^2 + eps) * scale: a wave a
+// (token, head).
+__global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, int64_t stride, int T, int heads,
+                                                         int d, float eps, float scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads), h = static_cast<int>(item - static_cast<int64_t>(t) * heads);
+  float* p = x + t * stride + static_cast<int64_t>(h) * d;
+  float ss = 0.f;
+  for (int i = lane; i < d; i += kWave) ss = fmaf(p[i], p[i], ss);
+  ss = wave_sum(ss);
+  const float inv = scale / sqrtf(ss + eps);
+  for (int i = lane; i < d; i += kWave) p[i] *= inv;
+}
+
+// out[t, h, c] = o[t, h, c] / sqrt(mean_c o^2 + eps) * gain[c] * silu(gate[t, h, c]): the norm of
+// every head first, then the gate.  A wave a (token, head).
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(
+    TO* __restrict__ out, const float* __restrict__ o, const TG* __restrict__ gate, int64_t gate_stride,
+    const float* __restrict__ gain, float eps, int T, int heads, int dv) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads), h = static_cast<int>(item - static_cast<int64_t>(t) * heads);
+  const float* p = o + (static_cast<int64_t>(t) * heads + h) * dv;
+  const TG* gp = gate + t * gate_stride + static_cast<int64_t>(h) * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += kWave) ss = fmaf(p[i], p[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(dv) + eps);
+  TO* op = out + (static_cast<int64_t>(t) * heads + h) * dv;
+  for (int i = lane; i < dv; i += kWave)
+    op[i] = from_float<TO>(p[i] * inv * gain[i] * silu_ff(to_float(gp[i])));
+}
+
+}  // namespace
+
+extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
+                                     int64_t k_stride, const float* v, int64_t v_stride,
+                                     const float* decay, int64_t decay_stride, const float* beta,
+                                     int64_t beta_stride, float* state, const int32_t* positions,
+                                     const int32_t* token_req, const int32_t* q_start,
+                                     const int32_t* slots, int R, int nh, int nqk, int d, int dv,
+                                     int delta_rule, float q_scale, kvc_stream stream) {
+  if (R < 0 || nh <= 0 || nqk <= 0 || nh % nqk || d <= 0 || dv <= 0)
+    return kvc_fail("kvc_linear_state_scan: bad sizes");
+  if (d > 256) return kvc_fail("kvc_linear_state_scan: at most 256 key channels a head");
+  if (delta_rule && beta == nullptr) return kvc_fail("kvc_linear_state_scan: the delta rule needs beta");
+  if (q_stride < static_cast<int64_t>(nqk) * d || k_stride < static_cast<int64_t>(nqk) * d ||
+      v_stride < static_cast<int64_t>(nh) * dv || decay_stride < (delta_rule ? nh : static_cast<int64_t>(nh) * d))
+    return kvc_fail("kvc_linear_state_scan: rows too short for the heads");
+  if (R == 0) return 0;
+  // tiles of 64 value channels with 4 threads a column, or, where that leaves compute units
+  // without a block, tiles of 16 with 16 threads a column
+  int VT = 64, NSL = 4;
+  const int64_t wide_blocks = static_cast<int64_t>(R) * nh * ((dv + 63) / 64);
+  if (dv < 64 || wide_blocks < kvc_device_compute_units()) {
+    VT = 16;
+    NSL = 16;
+  }
+  const dim3 grid(R, nh, (dv + VT - 1) / VT);
+  if (grid.y > 65535u || grid.z > 65535u) return kvc_fail("kvc_linear_state_scan: grid too large");
+  const dim3 block(VT * NSL);
+  const size_t lds = sizeof(float) * (2 * LSC * d + LSC * (delta_rule ? 2 : d) + LSC * VT);
+  const int per_thread = (d + NSL - 1) / NSL;
+#define KVC_LSCAN(NPT, DELTA)                                                                           \
+  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA>), grid, block, lds, S(stream), out, q, q_stride, \
+                     k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state, positions, \
+                     token_req, q_start, slots, nh, nqk, d, dv, VT, NSL, q_scale)
+#define KVC_LSCAN_N(NPT)        \
+  do {                          \
+    if (delta_rule) {           \
+      KVC_LSCAN(NPT, 1);        \
+    } else {                    \
+      KVC_LSCAN(NPT, 0);        \
+    }                           \
+  } while (0)
+  if (per_thread <= 8) {
+    KVC_LSCAN_N(8);
+  } else if (per_thread <= 16) {
+    KVC_LSCAN_N(16);
+  } else if (per_thread <= 32) {
+    KVC_LSCAN_N(32);
+  } else {
+    KVC_LSCAN_N(64);
+  }
+#undef KVC_LSCAN_N
+#undef KVC_LSCAN
+  return kvc_check_launch("kvc_linear_state_scan");
+}
+
+extern "C" int kvc_sigmoid_power(float* a, const float* z, int64_t z_stride, const float* bias,
+                                 float inv_tau, int T, int W, kvc_stream stream) {
+  if (T < 0 || W <= 0 || z_stride < W) return kvc_fail("kvc_sigmoid_power: bad sizes");
+  if (T == 0) return 0;
+  const int64_t n = static_cast<int64_t>(T) * W;
+  hipLaunchKernelGGL(sigmoid_power_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, S(stream),
+                     a, z, z_stride, bias, inv_tau, T, W);
+  return kvc_check_launch("kvc_sigmoid_power");
+}
+
+extern "C" int kvc_decay_and_write_gates(float* g, float* beta, const float* a_raw, int64_t a_stride,
+                                         const float* b_raw, int64_t b_stride, const float* a_log,
+                                         const float* dt_bias, int T, int nh, kvc_stream stream) {
+  if (T < 0 || nh <= 0 || a_stride < nh || b_stride < nh) return kvc_fail("kvc_decay_and_write_gates: bad sizes");
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(decay_and_write_gates_kernel, dim3((T * nh + 255) / 256), dim3(256), 0, S(stream), g, beta,
+                     a_raw, a_stride, b_raw, b_stride, a_log, dt_bias, T, nh);
+  return kvc_check_launch("kvc_decay_and_write_gates");
+}
+
+extern "C" int kvc_unit_heads(float* x, int64_t stride, int T, int heads, int d, float eps, float scale,
+                              kvc_stream stream) {
+  if (T < 0 || heads <= 0 || d <= 0 || stride < static_cast<int64_t>(heads) * d)
+    return kvc_fail("kvc_unit_heads: bad sizes");
+  if (T == 0) return 0;
+  const int64_t waves = static_cast<int64_t>(T) * heads;
+  hipLaunchKernelGGL(unit_heads_kernel, dim3(static_cast<unsigned>((waves + 3) / 4)), dim3(256), 0, S(stream), x,
+                     stride, T, heads, d, eps, scale);
+  return kvc_check_launch("kvc_unit_heads");
+}
+
+extern "C" int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* gate,
+                                     int64_t gate_stride, int gate_dtype, const float* gain, float eps,
+                                     int T, int heads, int dv, kvc_stream stream) {
+  if (T < 0 || heads <= 0 || dv <= 0 || gate_stride < static_cast<int64_t>(heads) * dv)
+    return kvc_fail("kvc_head_rmsnorm_gate: bad sizes");
+  if (T == 0) return 0;
+  const int64_t waves = static_cast<int64_t>(T) * heads;
+  const dim3 grid(static_cast<unsigned>((waves + 3) / 4));
+#define KVC_HRG(TG, TO)                                                                                  \
+  hipLaunchKernelGGL((head_rmsnorm_gate_kernel<TG, TO>), grid, dim3(256), 0, S(stream), static_cast<TO*>(out), o, \
+                     static_cast<const TG*>(gate), gate_stride, gain, eps, T, heads, dv)
+  if (gate_dtype == 0 && out_dtype == 0) {
+    KVC_HRG(float, float);
+  } else if (gate_dtype == 0 && out_dtype == 1) {
+    KVC_HRG(float, bf16_t);
+  } else if (gate_dtype == 1 && out_dtype == 1) {
+    KVC_HRG(bf16_t, bf16_t);
+  } else if (gate_dtype == 1 && out_dtype == 0) {
+    KVC_HRG(bf16_t, float);
+  } else {
+    return kvc_fail("kvc_head_rmsnorm_gate: unknown dtype code");
+  }
+#undef KVC_HRG
+  return kvc_check_launch("kvc_head_rmsnorm_gate");
+}

@@ -1,0 +1,394 @@
+// Routed experts: the router's choice, the arrangement of (token, choice) pairs by expert, the
+// experts' two products over their own rows, and the weighted sum.
+//
+// Everything is decided on the device and every grid is sized by bounds known on the host (pairs =
+// tokens x choices, tiles <= pairs / 16 + experts), so a step neither waits for the routing nor
+// changes its launches with it: a captured step replays for any routing.
+//
+//   kvc_moe_route    scores = softmax(logits) in float32; the `keep` groups whose best score is
+//                    highest; the `top` best experts of those groups (the lower index on a tie);
+//                    weights = chosen scores / (their sum + 1e-20).  A wave a token.
+//   kvc_moe_align    pairs sorted by expert: sorted[i] = pair index (token * top + choice), and a
+//                    list of tiles of up to 16 sorted rows that belong to one expert each.
+//   kvc_moe_gemm     for every tile, rows x that expert's matrix.  Gated: gate and up rows of the
+//                    expert side by side in one pass, and the activation
+//                    min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + 1) on the way out.
+//                    bfloat16 operands go through the matrix cores (16 x 16 x 32, the expert's rows as
+//                    the A operand, the tokens as B) with float32 sums; float32 operands are summed
+//                    in float32 in index order.  A row's sums do not depend on which tile it is in.
+//   kvc_moe_combine  out[t] = sum_c weight[t, c] * y[t * top + c] (+ up to two more row sets),
+//                    float32, in the order of the choices.
+//   kvc_clamped_glu  the same activation for a feed-forward that every token runs.
+
+#include <hip/hip_runtime.h>
+
+#include "device_utils.h"
+#include "gemm_common.h"
+#include "kvcore_hip.h"
+
+using namespace kvc;
+
+namespace {
+
+#define S(stream) reinterpret_cast<hipStream_t>(stream)
+
+constexpr int kTileRows = 16;
+
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+}
+
+// the lane that holds the largest value (the lowest index among equals) tells everyone
+__device__ __forceinline__ void wave_argmax(float& val, int& idx) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(val, o, kWave);
+    const int oi = __shfl_xor(idx, o, kWave);
+    if (ov > val || (ov == val && oi < idx)) {
+      val = ov;
+      idx = oi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
+                                                        const float* __restrict__ logits, int T, int E,
+                                                        int top, int groups, int keep) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  float* sc = lds + wave * (E + groups);  // scores, then the groups' best
+  float* gs = sc + E;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;  // the whole wave
+  const float* z = logits + static_cast<int64_t>(t) * E;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += kWave) {
+    const float p = expf(z[e] - mx);
+    sc[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int e = lane; e < E; e += kWave) sc[e] *= inv;
+  __builtin_amdgcn_wave_barrier();
+  const int per = E / groups;
+  if (keep < groups) {
+    for (int g = lane; g < groups; g += kWave) {
+      float best = -INFINITY;
+      for (int i = 0; i < per; ++i) best = fmaxf(best, sc[g * per + i]);
+      gs[g] = best;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // the best `keep` groups are marked with +inf; the others' experts are taken out
+    for (int r = 0; r < keep; ++r) {
+      float val = -INFINITY;
+      int idx = 0x7fffffff;
+      for (int g = lane; g < groups; g += kWave) {
+        const float s = gs[g];
+        if (s != INFINITY && (s > val || (s == val && g < idx))) {
+          val = s;
+          idx = g;
+        }
+      }
+      wave_argmax(val, idx);
+      if (lane == 0 && idx < groups) gs[idx] = INFINITY;
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int e = lane; e < E; e += kWave)
+      if (gs[e / per] != INFINITY) sc[e] = -1.f;  // scores are positive: never chosen before a kept one
+    __builtin_amdgcn_wave_barrier();
+  }
+  float total = 0.f;
+  float mine = 0.f;  // lane c keeps the c-th choice's score
+  int mine_idx = 0;
+  for (int c = 0; c < top; ++c) {
+    float val = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int e = lane; e < E; e += kWave) {
+      const float s = sc[e];
+      if (s > val || (s == val && e < idx)) {
+        val = s;
+        idx = e;
+      }
+    }
+    wave_argmax(val, idx);
+    if (idx >= E) { idx = 0; val = 0.f; }
+    if (val < 0.f) val = 0.f;  // fewer allowed experts than choices: a weight of zero
+    total += val;
+    if (lane == c) {
+      mine = val;
+      mine_idx = idx;
+    }
+    if (lane == 0) sc[idx] = -2.f;
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float norm = 1.f / (total + 1e-20f);
+  if (lane < top) {
+    choice[static_cast<int64_t>(t) * top + lane] = mine_idx;
+    weight[static_cast<int64_t>(t) * top + lane] = mine * norm;
+  }
+}
+
+// One block.  counts -> offsets -> sorted pairs -> tiles.
+__global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ sorted, int32_t* __restrict__ tiles,
+                                                         int32_t* __restrict__ num_tiles,
+                                                         const int32_t* __restrict__ choice, int pairs, int E,
+                                                         int max_tiles) {
+  extern __shared__ int32_t ilds[];
+  int32_t* count = ilds;           // [E]
+  int32_t* offset = count + E;     // [E + 1]
+  int32_t* cursor = offset + E + 1;  // [E]
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = choice[i];
+    if (e >= 0 && e < E) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      offset[e] = at;
+      cursor[e] = 0;
+      for (int r = 0; r < count[e] && nt < max_tiles; r += kTileRows, ++nt) {
+        tiles[3 * nt] = e;
+        tiles[3 * nt + 1] = at + r;
+        tiles[3 * nt + 2] = (count[e] - r < kTileRows) ? count[e] - r : kTileRows;
+      }
+      at += count[e];
+    }
+    offset[E] = at;
+    *num_tiles = nt;
+  }
+  __syncthreads();
+  // an expert's pairs take their places in the order in which their threads arrive: a row's sums
+  // do not depend on its place
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int e = choice[i];
+    if (e < 0 || e >= E) continue;
+    const int place = atomicAdd(&cursor[e], 1);
+    sorted[offset[e] + place] = i;
+  }
+}
+
+// bfloat16: a block of four waves takes one tile of rows and 64 columns (16 a wave).
+template <int GATED, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
+    TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
+    const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  if (n0 >= N) return;
+  const int li = lane & 15, lk = lane >> 4;
+  // B operand: token row li of the tile, 8 values of k from 8 * lk
+  const bool row_ok = li < nr;
+  const int pair = row_ok ? sorted[r0 + li] : 0;
+  const int64_t in_row = in_div > 0 ? pair / in_div : r0 + li;
+  const bf16_t* xr = x + in_row * x_stride + 8 * lk;
+  // A operand: the expert's row n0 + li
+  const int wrow = n0 + li < N ? n0 + li : N - 1;
+  const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* wr = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 8 * lk;
+  const bf16_t* wr2 = wr + static_cast<int64_t>(N) * K;  // the up rows follow the gate rows
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  const int k_main = K & ~31;
+  for (int k = 0; k < k_main; k += 32) {
+    bf16x8_t b = zero8();
+    if (row_ok) b = *reinterpret_cast<const bf16x8_t*>(xr + k);
+    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(wr + k);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    if (GATED) {
+      const bf16x8_t a2 = *reinterpret_cast<const bf16x8_t*>(wr2 + k);
+      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc2, 0, 0, 0);
+    }
+  }
+  if (k_main < K) {  // a ragged end along K: element by element, zeros beyond
+    bf16x8_t a = zero8(), a2 = zero8(), b = zero8();
+    for (int i = 0; i < 8; ++i) {
+      const int kk = k_main + 8 * lk + i;
+      if (kk < K) {
+        const __bf16* wp = reinterpret_cast<const __bf16*>(wr + k_main);
+        a[i] = wp[i];
+        if (GATED) a2[i] = reinterpret_cast<const __bf16*>(wr2 + k_main)[i];
+        if (row_ok) b[i] = reinterpret_cast<const __bf16*>(xr + k_main)[i];
+      }
+    }
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+    if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc2, 0, 0, 0);
+  }
+  // lane holds column (token) li, rows (features) n0 + 4 * lk + i
+  if (!row_ok) return;
+  if (GATED) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = clamped_glu(acc[i], acc2[i], limit, alpha);
+  }
+  const int64_t out_row = out_sorted ? r0 + li : pair;
+  const int nf = n0 + 4 * lk;
+  if (nf < N) store4<TO>(out + out_row * out_stride + nf, acc, N - nf);
+}
+
+// float32: a thread a (row, column) pair of the tile, sums in index order.
+template <int GATED>
+__global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
+    float* __restrict__ out, int64_t out_stride, const float* __restrict__ x, int64_t x_stride,
+    const float* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
+  const int li = threadIdx.x & 15, col = threadIdx.x >> 4;  // 16 rows x 16 columns a pass
+  if (li >= nr) return;
+  const int pair = sorted[r0 + li];
+  const int64_t in_row = in_div > 0 ? pair / in_div : r0 + li;
+  const float* xr = x + in_row * x_stride;
+  const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
+  const int64_t out_row = out_sorted ? r0 + li : pair;
+  for (int n = blockIdx.y * 64 + col; n < N && n < (blockIdx.y + 1) * 64; n += 16) {
+    const float* wr = w + (static_cast<int64_t>(e) * rows_per_expert + n) * K;
+    float acc = 0.f, acc2 = 0.f;
+    for (int k = 0; k < K; ++k) {
+      acc = fmaf(xr[k], wr[k], acc);
+      if (GATED) acc2 = fmaf(xr[k], wr[static_cast<int64_t>(N) * K + k], acc2);
+    }
+    out[out_row * out_stride + n] = GATED ? clamped_glu(acc, acc2, limit, alpha) : acc;
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
+                                                          const float* __restrict__ weight, int top,
+                                                          const TA* __restrict__ add0, const float* __restrict__ add1,
+                                                          int T, int H) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= static_cast<int64_t>(T) * H) return;
+  const int t = static_cast<int>(idx / H), c = static_cast<int>(idx - static_cast<int64_t>(t) * H);
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j)
+    acc = fmaf(weight[static_cast<int64_t>(t) * top + j], y[(static_cast<int64_t>(t) * top + j) * H + c], acc);
+  if (add0 != nullptr) acc += to_float(add0[idx]);
+  if (add1 != nullptr) acc += add1[idx];
+  out[idx] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ gate_up,
+                                                          int64_t n, int I, float limit, float alpha) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t t = idx / I, i = idx - t * I;
+  const T* row = gate_up + t * 2 * I;
+  out[idx] = from_float<T>(clamped_glu(to_float(row[i]), to_float(row[I + i]), limit, alpha));
+}
+
+}  // namespace
+
+extern "C" int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
+                             int groups, int keep, kvc_stream stream) {
+  if (T < 0 || E <= 0 || top <= 0 || top > E || top > kWave || groups <= 0 || E % groups || keep <= 0 ||
+      keep > groups)
+    return kvc_fail("kvc_moe_route: bad sizes (at most 64 choices; the experts in equal groups)");
+  const size_t lds = sizeof(float) * 4 * (E + groups);
+  if (lds > 60000) return kvc_fail("kvc_moe_route: too many experts for a wave's scores in LDS");
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), lds, S(stream), choice, weight, logits, T, E,
+                     top, groups, keep);
+  return kvc_check_launch("kvc_moe_route");
+}
+
+extern "C" int kvc_moe_max_tiles(int pairs, int E) { return (pairs + kTileRows - 1) / kTileRows + E; }
+
+extern "C" int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int32_t* choice,
+                             int pairs, int E, int max_tiles, kvc_stream stream) {
+  if (pairs < 0 || E <= 0 || max_tiles < kvc_moe_max_tiles(pairs, E))
+    return kvc_fail("kvc_moe_align: bad sizes, or room for fewer tiles than the routing may need");
+  const size_t lds = sizeof(int32_t) * (3 * E + 1);
+  if (lds > 60000) return kvc_fail("kvc_moe_align: too many experts");
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), lds, S(stream), sorted, tiles, num_tiles, choice,
+                     pairs, E, max_tiles);
+  return kvc_check_launch("kvc_moe_align");
+}
+
+extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
+                            const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
+                            const int32_t* num_tiles, int max_tiles, int N, int K, int in_div,
+                            int out_sorted, int gated, float limit, float alpha, kvc_stream stream) {
+  if (max_tiles < 0 || N <= 0 || K <= 0 || x_stride < K || out_stride < N)
+    return kvc_fail("kvc_moe_gemm: bad sizes");
+  if (max_tiles == 0) return 0;
+  const dim3 grid(max_tiles, (N + 63) / 64);
+  if (grid.y > 65535u) return kvc_fail("kvc_moe_gemm: too many columns");
+#define KVC_MOE_ARGS sorted, tiles, num_tiles, N, K, in_div, out_sorted, limit, alpha
+  if (dtype == 1) {
+    if (K % 8 || x_stride % 8 || (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(w) & 15))
+      return kvc_fail("kvc_moe_gemm: bfloat16 rows must be multiples of 8 values, 16-byte aligned");
+    const bf16_t* xb = static_cast<const bf16_t*>(x);
+    const bf16_t* wb = static_cast<const bf16_t*>(w);
+    if (gated && out_dtype == 1) {
+      hipLaunchKernelGGL((moe_gemm_bf16_kernel<1, bf16_t>), grid, dim3(256), 0, S(stream), static_cast<bf16_t*>(out),
+                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
+    } else if (gated && out_dtype == 0) {
+      hipLaunchKernelGGL((moe_gemm_bf16_kernel<1, float>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
+                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
+    } else if (out_dtype == 1) {
+      hipLaunchKernelGGL((moe_gemm_bf16_kernel<0, bf16_t>), grid, dim3(256), 0, S(stream), static_cast<bf16_t*>(out),
+                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
+    } else if (out_dtype == 0) {
+      hipLaunchKernelGGL((moe_gemm_bf16_kernel<0, float>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
+                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
+    } else {
+      return kvc_fail("kvc_moe_gemm: unknown dtype code");
+    }
+  } else if (dtype == 0) {
+    if (out_dtype != 0) return kvc_fail("kvc_moe_gemm: float32 operands give float32 rows");
+    if (gated) {
+      hipLaunchKernelGGL((moe_gemm_f32_kernel<1>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
+                         out_stride, static_cast<const float*>(x), x_stride, static_cast<const float*>(w),
+                         KVC_MOE_ARGS);
+    } else {
+      hipLaunchKernelGGL((moe_gemm_f32_kernel<0>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
+                         out_stride, static_cast<const float*>(x), x_stride, static_cast<const float*>(w),
+                         KVC_MOE_ARGS);
+    }
+  } else {
+    return kvc_fail("kvc_moe_gemm: unknown dtype code");
+  }
+#undef KVC_MOE_ARGS
+  return kvc_check_launch("kvc_moe_gemm");
+}
+
+extern "C" int kvc_moe_combine(float* out, const float* y, const float* weight, int top, const void* add0,
+                               int add0_dtype, const float* add1, int T, int H, kvc_stream stream) {
+  if (T < 0 || H <= 0 || top < 0) return kvc_fail("kvc_moe_combine: bad sizes");
+  if (T == 0) return 0;
+  const int64_t n = static_cast<int64_t>(T) * H;
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  if (add0_dtype == 1) {
+    hipLaunchKernelGGL((moe_combine_kernel<bf16_t>), grid, dim3(256), 0, S(stream), out, y, weight, top,
+                       static_cast<const bf16_t*>(add0), add1, T, H);
+  } else {
+    hipLaunchKernelGGL((moe_combine_kernel<float>), grid, dim3(256), 0, S(stream), out, y, weight, top,
+                       static_cast<const float*>(add0), add1, T, H);
+  }
+  return kvc_check_launch("kvc_moe_combine");
+}
+
+extern "C" int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, float limit, float alpha, int dtype,
+                               kvc_stream stream) {
+  if (T < 0 || I <= 0) return kvc_fail("kvc_clamped_glu: bad sizes");
+  if (T == 0) return 0;
+  const int64_t n = static_cast<int64_t>(T) * I;
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL((clamped_glu_kernel<Tp>), grid, dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(gate_up), n, I, limit, alpha));
+  return kvc_check_launch("kvc_clamped_glu");
+}

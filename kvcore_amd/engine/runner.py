@@ -74,6 +74,11 @@ def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.d
 
     config = config_override if config_override is not None else read_config_json(model_dir)
     arch = resolve_architecture(config)
+    if arch.complete_config is not None and load_format != "random":
+        from kvcore_amd.weights.safetensors_io import tensor_shapes
+
+        shapes = tensor_shapes(model_dir)  # sizes that only the checkpoint's tensors give
+        config = arch.complete_config(config, shapes.get)
     typed = arch.parse_config(config)
     spec = arch.build_spec(typed)
     model = DecoderModel(spec, dtype, device)
@@ -82,6 +87,7 @@ def build_model(model_dir: str | Path, dtype: torch.dtype, device: str | torch.d
         init_random_weights(model, seed)
     else:
         load_weights(model, model_dir, strict=strict)
+    model.weights_loaded()
     model.packed_bytes = model.pack_product_weights(pack_weights)
     return model
 

@@ -184,6 +184,11 @@ class DecoderModel:
             return {f"{self.spec.head_prefix}.weight"}
         return set()
 
+    def weights_loaded(self) -> None:
+        """Tell every part that its parameters hold their values now."""
+        for _, part in self._owned:
+            part.weights_loaded()
+
     def graph_safe(self) -> bool:
         """True iff every part says its forward may be captured into a HIP graph (it reads
         nothing from the device and decides nothing on the host per step)."""

@@ -40,13 +40,25 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_add_slices_rmsnorm": [P, P, P, I, P, P, F, I, I, I, P],
         "kvc_rmsnorm": [P, P, P, F, I, I, L, L, I, P],
         "kvc_residual_add": [P, P, I, I, I, P],
+        "kvc_residual_add2": [P, P, I, P, I, I, I, P],
         "kvc_silu_mul": [P, P, I, I, I, P],
         "kvc_gather_rows": [P, P, P, I, I, I, I, P],
         "kvc_to_float": [P, P, L, I, P],
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
-        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
+        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, I, P],
+        "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, P],
+        "kvc_sigmoid_power": [P, P, L, P, F, I, I, P],
+        "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
+        "kvc_unit_heads": [P, L, I, I, I, F, F, P],
+        "kvc_head_rmsnorm_gate": [P, I, P, P, L, I, P, F, I, I, I, P],
+        "kvc_moe_route": [P, P, P, I, I, I, I, I, P],
+        "kvc_moe_max_tiles": [I, I],
+        "kvc_moe_align": [P, P, P, P, I, I, I, P],
+        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, F, F, P],
+        "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, P],
+        "kvc_clamped_glu": [P, P, I, I, F, F, I, P],
         "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_add_layernorm": [P, P, P, P, P, F, I, I, I, P],
         "kvc_rms_branches_mean": [P, P, P, I, F, I, I, I, P],
@@ -254,6 +266,15 @@ def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> None:
                                    T, H, _code(delta, "delta"), _stream()), "kvc_residual_add")
 
 
+def residual_add2(residual: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
+    """``residual += a + b``, the two branches added to each other first."""
+    T, H = residual.shape
+    if a.shape != (T, H) or b.shape != (T, H):
+        raise KernelError("residual_add2: shapes do not match")
+    _check(load().kvc_residual_add2(_dev(residual, "residual", torch.float32), _dev(a, "a"), _code(a, "a"),
+                                    _dev(b, "b"), _code(b, "b"), T, H, _stream()), "kvc_residual_add2")
+
+
 def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> None:
     T, I2 = gate_up.shape
     if I2 % 2 or out.shape != (T, I2 // 2) or out.dtype != gate_up.dtype:
@@ -330,9 +351,14 @@ def rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
                     slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-                    window: int = 0, dv: int | None = None) -> None:
+                    window: int = 0, dv: int | None = None, slopes: torch.Tensor | None = None,
+                    chunk: int = 0) -> None:
     """``q`` is a ``[T, >= nh*d]`` view whose rows hold the query heads first.  ``dv``: the size
-    of a value head where it differs from a key head's ``d`` (``out`` is ``[T, nh*dv]``)."""
+    of a value head where it differs from a key head's ``d`` (``out`` is ``[T, nh*dv]``).
+    ``slopes`` (float32 ``[nh]``): ``slopes[h] * distance`` is taken off every score of head h;
+    ``chunk``: a token sees only the keys of its own chunk of that many positions."""
+    if slopes is not None and (slopes.shape != (nh,) or slopes.dtype != torch.float32):
+        raise KernelError("paged_attention: slopes must be float32 [nh]")
     T = out.shape[0]
     dv = d if dv is None else dv
     if out.shape != (T, nh * dv) or not out.is_contiguous():
@@ -349,7 +375,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         _dev(table, "table", torch.int32), table.shape[1],
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(slots, "slots", torch.int32), T, nh, nkv, d, dv, page_size, num_pages, float(scale),
-        int(window), _code(out, "out"), _stream()), "kvc_paged_attention")
+        int(window), None if slopes is None else _dev(slopes, "slopes"), int(chunk),
+        _code(out, "out"), _stream()), "kvc_paged_attention")
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor,
@@ -1193,6 +1220,167 @@ def gated_group_rmsnorm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, gai
         _dev(out, "out"), _code(out, "out"), _dev(y, "y", torch.float32), z_ptr, z_stride, z_code,
         _dev(gain, "gain", torch.float32), float(eps), T, width, groups, _stream()),
         "kvc_gated_group_rmsnorm")
+
+
+def _f32_rows(t: torch.Tensor, name: str, cols: int) -> tuple[int, int]:
+    ptr, stride, code = _rows(t, name, cols)
+    if code != 0:
+        raise KernelError(f"{name} must be float32")
+    return ptr, stride
+
+
+def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                      decay: torch.Tensor, beta: torch.Tensor | None, state: torch.Tensor, *,
+                      positions: torch.Tensor, token_req: torch.Tensor, q_start: torch.Tensor,
+                      slots: torch.Tensor, num_reqs: int, heads: int, qk_heads: int, dim: int,
+                      vdim: int, delta_rule: bool, q_scale: float = 1.0) -> None:
+    """The recurrence of a matrix state per head (see the C header): ``q, k [T, qk_heads * dim]``,
+    ``v [T, heads * vdim]``, all float32 rows (column views are fine); ``decay [T, heads * dim]``
+    (a factor per key channel) or, with ``delta_rule``, ``decay`` and ``beta [T, heads]``;
+    ``state [slots, heads, dim, vdim]`` float32; ``out [T, heads * vdim]`` float32.  ``q_scale``
+    multiplies every q on its way in."""
+    T = out.shape[0]
+    if out.shape != (T, heads * vdim) or not out.is_contiguous() or out.dtype != torch.float32:
+        raise KernelError("linear_state_scan: out must be contiguous float32 [T, heads * vdim]")
+    if tuple(state.shape[1:]) != (heads, dim, vdim) or state.dtype != torch.float32 or not state.is_contiguous():
+        raise KernelError("linear_state_scan: state must be float32 [slots, heads, dim, vdim]")
+    if min(q.shape[0], k.shape[0], v.shape[0], decay.shape[0]) < T or positions.numel() < T \
+            or token_req.numel() < T or q_start.numel() < num_reqs + 1:
+        raise KernelError("linear_state_scan: rows or index arrays too short")
+    qp, qs = _f32_rows(q, "q", qk_heads * dim)
+    kp, ks = _f32_rows(k, "k", qk_heads * dim)
+    vp, vs = _f32_rows(v, "v", heads * vdim)
+    dp, ds = _f32_rows(decay, "decay", heads if delta_rule else heads * dim)
+    bp, bs = (0, 0)
+    if delta_rule:
+        if beta is None or beta.shape[0] < T:
+            raise KernelError("linear_state_scan: the delta rule needs beta")
+        bp, bs = _f32_rows(beta, "beta", heads)
+    _check(load().kvc_linear_state_scan(
+        out.data_ptr(), qp, qs, kp, ks, vp, vs, dp, ds, bp or None, bs, _dev(state, "state"),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, heads,
+        qk_heads, dim, vdim, int(bool(delta_rule)), float(q_scale), _stream()), "kvc_linear_state_scan")
+
+
+def sigmoid_power(out: torch.Tensor, z: torch.Tensor, bias: torch.Tensor | None, inv_tau: float) -> None:
+    """``out = sigmoid(z + bias) ** inv_tau`` in float32 (through the logarithm)."""
+    T, W = out.shape
+    if not out.is_contiguous() or out.dtype != torch.float32 or z.shape[0] < T or (bias is not None and bias.shape != (W,)):
+        raise KernelError("sigmoid_power: shapes do not match")
+    zp, zs = _f32_rows(z, "z", W)
+    _check(load().kvc_sigmoid_power(out.data_ptr(), zp, zs, None if bias is None else _dev(bias, "bias", torch.float32),
+                                    float(inv_tau), T, W, _stream()), "kvc_sigmoid_power")
+
+
+def decay_and_write_gates(g: torch.Tensor, beta: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor,
+                          a_log: torch.Tensor, dt_bias: torch.Tensor) -> None:
+    """``g = exp(-exp(a_log) * softplus(a_raw + dt_bias))``, ``beta = sigmoid(b_raw)``, float32 ``[T, heads]``."""
+    T, nh = g.shape
+    if beta.shape != (T, nh) or a_log.shape != (nh,) or dt_bias.shape != (nh,) or a_raw.shape[0] < T or b_raw.shape[0] < T:
+        raise KernelError("decay_and_write_gates: shapes do not match")
+    ap, as_ = _f32_rows(a_raw, "a_raw", nh)
+    bp, bs = _f32_rows(b_raw, "b_raw", nh)
+    f = torch.float32
+    _check(load().kvc_decay_and_write_gates(_dev(g, "g", f), _dev(beta, "beta", f), ap, as_, bp, bs,
+                                            _dev(a_log, "a_log", f), _dev(dt_bias, "dt_bias", f), T, nh, _stream()),
+           "kvc_decay_and_write_gates")
+
+
+def unit_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0) -> None:
+    """Every head of ``dim`` values of the float32 rows ``x [T, heads * dim]`` (a column view is
+    fine) over its Euclidean length (``eps`` inside the root), times ``scale``, in place."""
+    xp, xs = _f32_rows(x, "x", heads * dim)
+    _check(load().kvc_unit_heads(xp, xs, x.shape[0], heads, dim, float(eps), float(scale), _stream()),
+           "kvc_unit_heads")
+
+
+def head_rmsnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps: float,
+                      heads: int, vdim: int) -> None:
+    """``out = o / rms_head(o) * gain * silu(gate)``: every head of ``vdim`` values of the float32
+    ``o [T, heads * vdim]`` over its root mean square, times ``gain [vdim]`` (shared by the heads),
+    times the gate (rows of any dtype, a column view is fine)."""
+    T = o.shape[0]
+    if o.shape != (T, heads * vdim) or out.shape != o.shape or not out.is_contiguous() or not o.is_contiguous() \
+            or gain.shape != (vdim,):
+        raise KernelError("head_rmsnorm_gate: shapes do not match")
+    gp, gs, gc = _rows(gate, "gate", heads * vdim)
+    _check(load().kvc_head_rmsnorm_gate(_dev(out, "out"), _code(out, "out"), _dev(o, "o", torch.float32), gp, gs, gc,
+                                        _dev(gain, "gain", torch.float32), float(eps), T, heads, vdim, _stream()),
+           "kvc_head_rmsnorm_gate")
+
+
+def moe_route(choice: torch.Tensor, weight: torch.Tensor, logits: torch.Tensor, *, top: int, groups: int = 1,
+              keep: int = 1) -> None:
+    """The router's choice from float32 ``logits [T, E]``: ``choice`` (int32) and ``weight``
+    (float32), both ``[T, top]`` (see the C header for the rule)."""
+    T, E = logits.shape
+    if choice.shape != (T, top) or weight.shape != (T, top):
+        raise KernelError("moe_route: shapes do not match")
+    _check(load().kvc_moe_route(_dev(choice, "choice", torch.int32), _dev(weight, "weight", torch.float32),
+                                _dev(logits, "logits", torch.float32), T, E, top, groups, keep, _stream()),
+           "kvc_moe_route")
+
+
+def moe_max_tiles(pairs: int, experts: int) -> int:
+    return int(load().kvc_moe_max_tiles(pairs, experts))
+
+
+def moe_align(sorted_pairs: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, choice: torch.Tensor,
+              experts: int) -> None:
+    """(token, choice) pairs sorted by expert, and the list of row tiles (``tiles [>= max_tiles, 3]``)."""
+    pairs = choice.numel()
+    if sorted_pairs.numel() < pairs or tiles.dim() != 2 or tiles.shape[1] != 3 or num_tiles.numel() < 1:
+        raise KernelError("moe_align: buffers too small")
+    _check(load().kvc_moe_align(_dev(sorted_pairs, "sorted", torch.int32), _dev(tiles, "tiles", torch.int32),
+                                _dev(num_tiles, "num_tiles", torch.int32), _dev(choice, "choice", torch.int32),
+                                pairs, experts, tiles.shape[0], _stream()), "kvc_moe_align")
+
+
+def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tiles: torch.Tensor,
+             num_tiles: torch.Tensor, *, pairs: int, experts: int, in_div: int, out_sorted: bool, gated: bool,
+             limit: float = 0.0, alpha: float = 0.0) -> None:
+    """Every expert's product over its own rows.  ``w`` is ``[experts * N, K]`` (``experts * 2N``
+    rows when ``gated``: each expert's gate rows, then its up rows); ``out [pairs, N]``."""
+    N = out.shape[1]
+    K = x.shape[1]
+    rows = experts * N * (2 if gated else 1)
+    if w.shape != (rows, K) or out.shape[0] < pairs or x.dtype != w.dtype or out.stride(1) != 1 or x.stride(1) != 1:
+        raise KernelError("moe_gemm: shapes do not match")
+    max_tiles = min(tiles.shape[0], moe_max_tiles(pairs, experts))
+    _check(load().kvc_moe_gemm(out.data_ptr(), out.stride(0), _code(out, "out"), x.data_ptr(), x.stride(0),
+                               _dev(w, "w"), _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
+                               _dev(tiles, "tiles", torch.int32), _dev(num_tiles, "num_tiles", torch.int32),
+                               max_tiles, N, K, int(in_div), int(bool(out_sorted)), int(bool(gated)),
+                               float(limit), float(alpha), _stream()), "kvc_moe_gemm")
+
+
+def moe_combine(out: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, add0: torch.Tensor | None = None,
+                add1: torch.Tensor | None = None) -> None:
+    """``out[t] = sum_c weight[t, c] * y[t * top + c] (+ add0[t]) (+ add1[t])``, float32; ``add0``
+    of either dtype, ``add1`` float32."""
+    T, H = out.shape
+    top = weight.shape[1] if weight.dim() == 2 else 0
+    if out.dtype != torch.float32 or (top and (y.shape[0] < T * top or y.shape[1] != H)):
+        raise KernelError("moe_combine: shapes do not match")
+    for a in (add0, add1):
+        if a is not None and a.shape != (T, H):
+            raise KernelError("moe_combine: an added row set does not fit")
+    _check(load().kvc_moe_combine(_dev(out, "out"), _dev(y, "y", torch.float32), _dev(weight, "weight", torch.float32),
+                                  top, None if add0 is None else _dev(add0, "add0"),
+                                  0 if add0 is None else _code(add0, "add0"),
+                                  None if add1 is None else _dev(add1, "add1", torch.float32), T, H, _stream()),
+           "kvc_moe_combine")
+
+
+def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, limit: float, alpha: float) -> None:
+    """``out = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up,
+    -limit, limit)`` from ``gate_up [T, 2I]`` (gate columns first)."""
+    T, I = out.shape
+    if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError("clamped_glu: shapes do not match")
+    _check(load().kvc_clamped_glu(_dev(out, "out"), _dev(gate_up, "gate_up"), T, I, float(limit), float(alpha),
+                                  _code(out, "out"), _stream()), "kvc_clamped_glu")
 
 
 def table_update(table: torch.Tensor, triples: torch.Tensor, n: int) -> None:

@@ -106,14 +106,19 @@ class PagedAttention(Mixer):
                  scale: float, bias: bool = False, window: int = 0, page_size: int | None = None,
                  v_head_dim: int | None = None, qk_norm_eps: float | None = None,
                  tensor_names: dict[str, str] | None = None, float32_result: bool = False,
-                 position: PositionEncoding | None = None) -> None:
+                 qk_norm_gain: bool = True, distance_slopes: tuple[float, ...] | None = None,
+                 chunk: int = 0, position: PositionEncoding | None = None) -> None:
         """``v_head_dim``: the size of a value head where it differs from ``head_dim``, the
         size of a query and key head.  ``qk_norm_eps`` (None: no such norm): every query and
         key head is divided by its root mean square, eps inside the root, and multiplied by a
         gain of ``head_dim`` values shared by all heads, before the rotation.  ``tensor_names``
         renames checkpoint tensors (keys ``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``;
         values relative to the part's prefix).  ``float32_result``: the output rows are
-        float32 sums, for a consumer that normalises them."""
+        float32 sums, for a consumer that normalises them.  ``qk_norm_gain`` False: the norm of
+        the heads has no gain (and no tensors).  ``distance_slopes``: a value per query head;
+        ``slope * (i - j)`` is taken off the score of query i and key j before the softmax (no
+        rotation is needed for such a layer).  ``chunk`` > 0: query i sees key j <= i only if
+        both lie in the same chunk of that many positions, counted from the sequence's start."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         v_head_dim = head_dim if v_head_dim is None else v_head_dim
@@ -128,6 +133,13 @@ class PagedAttention(Mixer):
         self.head_dim = head_dim
         self.v_head_dim = v_head_dim
         self.qk_norm_eps = qk_norm_eps
+        self.qk_norm_gain = bool(qk_norm_gain)
+        if distance_slopes is not None and len(distance_slopes) != num_heads:
+            raise ValueError(f"{len(distance_slopes)} distance slopes for {num_heads} heads")
+        if chunk < 0:
+            raise ValueError(f"a chunk of {chunk} positions")
+        self.distance_slopes = None if distance_slopes is None else tuple(float(v) for v in distance_slopes)
+        self.chunk = int(chunk)
         self.scale = scale
         self.bias = bias
         self.window = window
@@ -170,11 +182,19 @@ class PagedAttention(Mixer):
                                    sources=stacked("q_bias", "k_bias", "v_bias")))
             specs.append(ParamSpec("o_proj.bias", (self.hidden_size,), init="zeros",
                                    sources=(ParamSource(n["o_bias"], 0, self.hidden_size),)))
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_gain:
             for key in ("q_norm", "k_norm"):
                 specs.append(ParamSpec(key, (self.head_dim,), kind="vector", init="gain",
                                        sources=(ParamSource(n[key], 0, self.head_dim),)))
         return specs
+
+    def setup(self, runtime) -> None:
+        super().setup(runtime)
+        self._slopes = self._unit_gain = None
+        if self.distance_slopes is not None:
+            self._slopes = torch.tensor(self.distance_slopes, dtype=torch.float32, device=runtime.device)
+        if self.qk_norm_eps is not None and not self.qk_norm_gain:
+            self._unit_gain = torch.ones(self.head_dim, dtype=torch.float32, device=runtime.device)
 
     def cache_need(self) -> CacheNeed:
         values = ((self.num_kv_heads, self.v_plane_dim),) * self.v_planes
@@ -237,7 +257,7 @@ class PagedAttention(Mixer):
             ops.qk_norm_rope_kv_write(qkv, k_cache, v_planes, cos, sin, rot_dim=rot_dim,
                                       interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
                                       nkv=self.num_kv_heads, d=self.head_dim, dv=self.v_head_dim,
-                                      q_gain=p.get("q_norm"), k_gain=p.get("k_norm"),
+                                      q_gain=p.get("q_norm", self._unit_gain), k_gain=p.get("k_norm", self._unit_gain),
                                       eps=self.qk_norm_eps or 0.0, write_kv=call.write_cache)
             rot_dim, interleaved = 0, False
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
@@ -271,7 +291,11 @@ class PagedAttention(Mixer):
                       slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
                       scale=self.scale, window=self.window)
         x_dtype = qkv.dtype
-        if not self._same_sizes():
+        if self._slopes is not None or self.chunk > 0:
+            # scores with a distance bias or a chunked view: the general kernel
+            ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_plane_dim, slopes=self._slopes,
+                                chunk=self.chunk, **common)
+        elif not self._same_sizes():
             ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_plane_dim, **common)
         elif ctx.max_query_len == 1 and ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x_dtype):

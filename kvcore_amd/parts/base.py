@@ -166,6 +166,11 @@ class Part:
         """``params`` maps the local names of ``param_specs`` to device tensors."""
         self.params = params
 
+    def weights_loaded(self) -> None:
+        """Called whenever the parameters have received their values (from a checkpoint or at
+        random): a part that keeps tensors derived from them (a gain stored as its distance
+        from one, say) makes them here."""
+
 
 class Norm(Part):
     """``forward_fused`` adds ``delta`` (may be None) into the float32 ``residual`` in

@@ -101,4 +101,40 @@ class PreNormBlock(Block):
         return self.ffn.forward(x2, ctx, call)
 
 
+class ParallelResidualBlock(Block):
+    """``r += delta; h = norm(r); r += mixer(h) + ffn(h)``: one norm a layer, both branches read
+    its output, and both sums go straight into the float32 stream (nothing stays pending, so the
+    branches may hand over float32 rows).  With a feed-forward of kind ``none`` the mixer is
+    the layer."""
+
+    def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm],
+                 mixer_name: str = "mixer", ffn_name: str = "mlp", norm: str | None = None) -> None:
+        super().__init__(mixer=mixer, ffn=ffn, norms=norms)
+        self.norm_name = norm if norm is not None else next(iter(norms), None)
+        if self.norm_name not in norms:
+            raise ValueError(f"a parallel block needs its one norm; asked for {norm!r}, given {list(norms)}")
+        self.mixer_only = bool(getattr(ffn, "absent", False))
+        self.mixer_name, self.ffn_name = mixer_name, ffn_name
+
+    def children(self) -> dict[str, Part]:
+        out = {self.norm_name: self.norms[self.norm_name], self.mixer_name: self.mixer}
+        if not self.mixer_only:
+            out[self.ffn_name] = self.ffn
+        return out
+
+    def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
+        if isinstance(delta, (ops.ScaledRows, ops.NormedRows)):
+            raise RuntimeError("a parallel block takes its input from the stream, not from folded norms")
+        x = ctx.buf("block_x", residual.shape[1])
+        self.norms[self.norm_name].forward_fused(x, residual, delta)
+        a = self.mixer.forward(x, ctx, call)
+        if self.mixer_only:
+            ops.residual_add(residual, a)
+        else:
+            f = self.ffn.forward(x, ctx, call)
+            ops.residual_add2(residual, a, f)
+        return None
+
+
 register_block("prenorm", PreNormBlock)
+register_block("parallel_residual", ParallelResidualBlock)

@@ -1,0 +1,115 @@
+"""A feed-forward of routed experts: every token runs the few experts its router chooses.
+
+    scores = softmax(W_r h)                               (float32)
+    choice = the `top` best experts among those of the `keep` best of `groups` equal groups of
+             neighbouring experts (a group is as good as its best expert)
+    weight = scores[choice] / (sum of them + 1e-20)
+    out    = sum_c weight_c * expert_choice_c(h)  (+ shared(h), an expert that every token runs)
+
+An expert is a gated feed-forward with a clamped activation: ``g = min(W_gate h, limit)``, ``u =
+clamp(W_up h, -limit, limit)``, ``W_down (g * sigmoid(alpha g) * (u + 1))``.  The experts' matrices are
+stacked along a leading expert dimension (each expert's gate rows, then its up rows), the routing
+stays on the device and every launch is sized by the step's token count alone, so a step may be
+captured into a graph.  The result is float32 rows: the weighted sum is not rounded before it
+joins the stream.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kvcore_amd.ops import library as ops
+
+from .base import FeedForward, ParamSource, ParamSpec, register_feed_forward
+
+GLU_ALPHA = 1.702
+
+
+class RoutedExperts(FeedForward):
+    """``experts`` experts of ``expert_size`` hidden units, ``top`` a token; ``groups`` and
+    ``keep`` as above (1 and 1: every expert may be chosen); ``shared_size`` > 0 adds the shared
+    expert (``shared_limit`` its clamp).  ``tensor_names`` renames checkpoint tensors (keys:
+    router, expert (a pattern with ``{e}``), shared, gate, up, down)."""
+
+    def __init__(self, *, hidden_size: int, experts: int, top: int, expert_size: int, limit: float,
+                 groups: int = 1, keep: int = 1, shared_size: int = 0, shared_limit: float | None = None,
+                 alpha: float = GLU_ALPHA, tensor_names: dict[str, str] | None = None) -> None:
+        if experts <= 0 or not 0 < top <= experts or expert_size <= 0:
+            raise ValueError(f"{top} of {experts} experts of {expert_size} units")
+        if groups <= 0 or experts % groups or not 0 < keep <= groups:
+            raise ValueError(f"{experts} experts do not form {groups} equal groups of which {keep} are kept")
+        if top > 64:
+            raise ValueError("the routing kernel serves at most 64 choices a token")
+        self.hidden_size, self.experts, self.top, self.expert_size = hidden_size, experts, top, expert_size
+        self.limit, self.groups, self.keep, self.alpha = float(limit), groups, keep, float(alpha)
+        self.shared_size = shared_size
+        self.shared_limit = float(limit if shared_limit is None else shared_limit)
+        self.names = {"router": "router.weight", "expert": "experts.{e}", "shared": "shared",
+                      "gate": "gate.weight", "up": "up.weight", "down": "down.weight", **(tensor_names or {})}
+
+    def param_specs(self) -> list[ParamSpec]:
+        n, H, E, I = self.names, self.hidden_size, self.experts, self.expert_size
+        gate_up, down = [], []
+        for e in range(E):
+            prefix = n["expert"].format(e=e)
+            gate_up.append(ParamSource(f"{prefix}.{n['gate']}", 2 * I * e, I))
+            gate_up.append(ParamSource(f"{prefix}.{n['up']}", 2 * I * e + I, I))
+            down.append(ParamSource(f"{prefix}.{n['down']}", H * e, H))
+        specs = [
+            ParamSpec("router.weight", (E, H), kind="vector", init="normal", sources=(ParamSource(n["router"], 0, E),)),
+            ParamSpec("experts.gate_up", (2 * I * E, H), sources=tuple(gate_up)),
+            ParamSpec("experts.down", (H * E, I), sources=tuple(down)),
+        ]
+        if self.shared_size:
+            S, sp = self.shared_size, n["shared"]
+            specs.append(ParamSpec("shared.gate_up", (2 * S, H), sources=(
+                ParamSource(f"{sp}.{n['gate']}", 0, S), ParamSource(f"{sp}.{n['up']}", S, S))))
+            specs.append(ParamSpec("shared.down", (H, S), sources=(ParamSource(f"{sp}.{n['down']}", 0, H),)))
+        return specs
+
+    def product_weights(self) -> tuple[str, ...]:
+        return ("shared.gate_up", "shared.down") if self.shared_size else ()
+
+    def forward(self, x, ctx, call, sink=None):
+        p, H, E, I, top = self.params, self.hidden_size, self.experts, self.expert_size, self.top
+        T = ctx.num_tokens
+        pairs = T * top
+        # the router reads the rows in float32 (of bfloat16 rows, their values as they are)
+        if x.dtype == torch.float32:
+            xf = x
+        else:
+            xf = ctx.buf(f"moe_x_f32:{H}", H, torch.float32)
+            ops.to_float(xf, x)
+        logits = ctx.buf(f"moe_logits:{E}", E, torch.float32)
+        ops.gemm_f32(logits, xf, p["router.weight"], None)
+        choice = ctx.buf(f"moe_choice:{top}", top, torch.int32)
+        weight = ctx.buf(f"moe_weight:{top}", top, torch.float32)
+        ops.moe_route(choice, weight, logits, top=top, groups=self.groups, keep=self.keep)
+        cap = ctx.buffers.token_capacity
+        sorted_pairs = ctx.buffers.get(f"moe_sorted:{top}", pairs, 1, torch.int32, reserve=cap * top).view(-1)
+        max_tiles = ops.moe_max_tiles(pairs, E)
+        tiles = ctx.buffers.get(f"moe_tiles:{top}:{E}", max_tiles, 3, torch.int32,
+                                reserve=ops.moe_max_tiles(cap * top, E))
+        num_tiles = ctx.buffers.get("moe_num_tiles", 1, 1, torch.int32).view(-1)
+        ops.moe_align(sorted_pairs, tiles, num_tiles, choice, E)
+        act = ctx.buffers.get(f"moe_act:{I}", pairs, I, ctx.dtype, reserve=cap * top)
+        ops.moe_gemm(act, x, p["experts.gate_up"], sorted_pairs, tiles, num_tiles, pairs=pairs, experts=E,
+                     in_div=top, out_sorted=True, gated=True, limit=self.limit, alpha=self.alpha)
+        y = ctx.buffers.get(f"moe_y:{H}", pairs, H, torch.float32, reserve=cap * top)
+        ops.moe_gemm(y, act, p["experts.down"], sorted_pairs, tiles, num_tiles, pairs=pairs, experts=E,
+                     in_div=0, out_sorted=False, gated=False)
+        shared = None
+        if self.shared_size:
+            S = self.shared_size
+            gate_up = ctx.buf(f"moe_shared_gu:{2 * S}", 2 * S)
+            ops.linear(gate_up, x, p["shared.gate_up"])
+            sact = ctx.buf(f"moe_shared_act:{S}", S)
+            ops.clamped_glu(sact, gate_up, self.shared_limit, self.alpha)
+            shared = ctx.buf(f"moe_shared_out:{H}", H, torch.float32)
+            ops.linear(shared, sact, p["shared.down"])
+        out = ctx.buf("ffn_out_f32", H, torch.float32)
+        ops.moe_combine(out, y, weight, shared, None)
+        return out
+
+
+register_feed_forward("routed_experts", RoutedExperts)

@@ -19,6 +19,9 @@ class Architecture:
     name: str
     parse_config: Callable[[Mapping[str, Any]], Any]
     build_spec: Callable[[Any], ModelSpec]
+    # fills in what config.json leaves to the checkpoint's tensor shapes: (config mapping, a
+    # function from tensor name to shape or None) -> config mapping; None: nothing to fill in
+    complete_config: Callable[[Mapping[str, Any], Callable[[str], Any]], Mapping[str, Any]] | None = None
 
 
 MODEL_REGISTRY: dict[str, Architecture] = {}
@@ -26,8 +29,8 @@ MODEL_REGISTRY: dict[str, Architecture] = {}
 
 def register_architecture(name: str, parse_config: Callable[[Mapping[str, Any]], Any],
                           build_spec: Callable[[Any], ModelSpec], *, aliases: tuple[str, ...] = (),
-                          replace: bool = False) -> None:
-    arch = Architecture(name, parse_config, build_spec)
+                          replace: bool = False, complete_config=None) -> None:
+    arch = Architecture(name, parse_config, build_spec, complete_config)
     for key in (name, *aliases):
         if key in MODEL_REGISTRY and not replace:
             raise ValueError(f"architecture {key!r} is already registered")
@@ -62,6 +65,12 @@ def _register_builtin() -> None:
     from kvcore_amd.models.dirulorn import dirulorn_spec
 
     register_architecture("Dirulorn", DirulornConfig.from_dict, dirulorn_spec)
+
+    from kvcore_amd.config.vovalix_config import VovalixConfig, complete_from_tensor_shapes
+    from kvcore_amd.models.vovalix import vovalix_spec
+
+    register_architecture("Vovalix", VovalixConfig.from_dict, vovalix_spec,
+                          complete_config=complete_from_tensor_shapes)
 
 
 _register_builtin()

@@ -169,6 +169,16 @@ def weight_files(model_dir: str | Path) -> list[Path]:
     return files
 
 
+def tensor_shapes(model_dir: str | Path) -> dict[str, tuple[int, ...]]:
+    """Name -> shape of every tensor in the folder's weight files, from their headers alone."""
+    shapes: dict[str, tuple[int, ...]] = {}
+    for path in weight_files(model_dir):
+        with SafetensorsFile(path) as f:
+            for name, entry in f.entries.items():
+                shapes[name] = tuple(entry.shape)
+    return shapes
+
+
 def iter_tensors(model_dir: str | Path) -> Iterator[tuple[str, torch.Tensor, SafetensorsFile]]:
     for path in weight_files(model_dir):
         if not path.is_file():
