@@ -179,11 +179,34 @@ def route(scores: torch.Tensor, top: int, groups: int, keep: int) -> tuple[list[
     return chosen, weights / (weights.sum() + 1e-20)
 
 
-def moe_feed_forward(x: torch.Tensor, w: dict, p: str, mlp: dict) -> torch.Tensor:
+def route_margin(logits: torch.Tensor, top: int, groups: int, keep: int) -> float:
+    """How far the router's choice for ``logits [E]`` is from another one: the smallest gap, in
+    units of the logits' spread, between a group that is kept and one that is not, and between an
+    expert that is chosen and an allowed one that is not (infinite where there is no other choice)."""
+    E = logits.shape[0]
+    per = E // groups
+    spread = float(logits.std()) if E > 1 else 1.0
+    gaps = [float("inf")]
+    best = [float(logits[g * per:(g + 1) * per].max()) for g in range(groups)]
+    ranked = sorted(range(groups), key=lambda g: (-best[g], g))
+    if keep < groups:
+        gaps.append(best[ranked[keep - 1]] - best[ranked[keep]])
+    allowed = sorted((float(logits[e]) for e in range(E) if e // per in set(ranked[:keep])), reverse=True)
+    if top < len(allowed):
+        gaps.append(allowed[top - 1] - allowed[top])
+    return min(gaps) / (spread + 1e-30)
+
+
+def moe_feed_forward(x: torch.Tensor, w: dict, p: str, mlp: dict, margins: list | None = None) -> torch.Tensor:
+    """``margins``, if given, receives a tensor ``[T]`` of every token's ``route_margin``."""
     r = mlp["router"]
     groups = r.get("groups") or {"count": 1, "keep": 1}
     limit = float(mlp["expert"]["limit"])
-    scores = torch.softmax(x @ w[f"{p}.router"].T, dim=-1)
+    logits = x @ w[f"{p}.router"].T
+    scores = torch.softmax(logits, dim=-1)
+    if margins is not None:
+        margins.append(torch.tensor([route_margin(logits[t], r["top"], groups["count"], groups["keep"])
+                                     for t in range(x.shape[0])], dtype=torch.float64))
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
         chosen, weights = route(scores[t], r["top"], groups["count"], groups["keep"])
@@ -199,9 +222,10 @@ MIXERS = {"attention": attention_mixer, "gla": gla_mixer, "delta": delta_mixer}
 
 
 def vovalix_forward(config: dict, weights: dict, tokens: list[int], dtype=torch.float64,
-                    return_layers: bool = False):
+                    return_layers: bool = False, margins: list | None = None):
     """Logits ``[T, vocab]`` of one sequence from position 0 (and, on request, the stream after
-    every layer run, ``[runs, T, width]``)."""
+    every layer run, ``[runs, T, width]``).  ``margins``, if given, receives one tensor ``[T]`` per
+    routed feed-forward: how clear each token's routing was (``route_margin``)."""
     w = {k: v.to(dtype) for k, v in weights.items()}
     eps = float(config["norm"]["eps"])
     x = w["embed"][torch.tensor(tokens)]
@@ -211,7 +235,7 @@ def vovalix_forward(config: dict, weights: dict, tokens: list[int], dtype=torch.
         h = offset_rms_norm(x, w[f"{p}.norm1"], eps)
         y = MIXERS[layer["type"]](h, w, f"{p}.mix", layer["mixer"], eps)
         if layer.get("mlp") is not None:
-            y = y + moe_feed_forward(h, w, f"{p}.mlp", layer["mlp"])
+            y = y + moe_feed_forward(h, w, f"{p}.mlp", layer["mlp"], margins)
         x = x + y
         seen.append(x)
     logits = offset_rms_norm(x, w["final.norm"], eps) @ w["embed"].T * float(config.get("logit_scale", 1.0))
