@@ -160,15 +160,18 @@ class VovalixConfig:
             kind = raw.get("type")
             if kind not in _MIXERS:
                 raise ConfigError(f"config.json: {where}type {kind!r} is not supported (supported: {sorted(_MIXERS)})")
-            mixer = _MIXERS[kind].from_dict(_mapping(raw, "mixer", where), where + "mixer.")
-            mlp = None if raw.get("mlp") is None else RoutedFeedForwardConfig.from_dict(raw["mlp"], where + "mlp.")
             source = raw.get("weights_of")
-            if source is not None:
+            if source is None:
+                mixer = _MIXERS[kind].from_dict(_mapping(raw, "mixer", where), where + "mixer.")
+                mlp = None if raw.get("mlp") is None else RoutedFeedForwardConfig.from_dict(raw["mlp"], where + "mlp.")
+            else:
                 source = int(source)
-                if not 0 <= source < i or layers[source].weights_of is not None:
-                    raise ConfigError(f"config.json: {where}weights_of must name an earlier layer with tensors of its own")
-                if (layers[source].type, layers[source].mixer, layers[source].mlp) != (kind, mixer, mlp):
-                    raise ConfigError(f"config.json: {where}differs from layer {source}, whose tensors it uses")
+                if not 0 <= source < i:
+                    raise ConfigError(f"config.json: {where}weights_of must name an earlier layer")
+                if layers[source].weights_of is not None:  # a layer that borrows in turn: its owner
+                    source = layers[source].weights_of
+                # the tensors are the owner's, so the owner's sizes are the ones that count
+                kind, mixer, mlp = layers[source].type, layers[source].mixer, layers[source].mlp
             layers.append(VovalixLayerConfig(kind, mixer, mlp, source))
         eos = d.get("eos_token_id")
         eos_ids = () if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos]))

@@ -69,6 +69,8 @@ struct DecodeArgs {
   int nh, nkv, page_size, num_pages;
   float scale_log2e;
   int window;
+  const float* slopes;  // [nh] or null: slope * (position - key position) comes off the score
+  int chunk;            // > 0: only the keys of the token's own chunk of so many positions
   int nsplit;
   int lds_pages;  // page ids of a block's range that fit in LDS
 };
@@ -106,6 +108,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   const int quad = lane >> 4;  // 0..3
   const int nh = a.nh, nkv = a.nkv, nsplit = a.nsplit, page_size = a.page_size;
   const int g = nh / nkv;
+  const float slope_l2e = (a.slopes != nullptr && col < g) ? a.slopes[hk * g + col] * kLog2e : 0.f;
   const bool head_live = col < g;
   constexpr int NJ = D / 16;  // output row blocks
   constexpr int NC = D / 32;  // 32-wide chunks of the head for Q.K
@@ -140,7 +143,8 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
     return;
   }
   const int window = a.window;
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (a.chunk > 0 && (pos / a.chunk) * a.chunk > first) first = (pos / a.chunk) * a.chunk;
   const int32_t* row = a.table + static_cast<int64_t>(trow_idx) * a.table_stride;
 
   // the 16-key blocks this block owns: [b0, b1) of the range that holds keys first..pos
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
     for (int i = 0; i < 4; ++i) {
       const int key = key0 + i;
       ok[i] = key >= first && key <= pos;
-      sv4[i] = ok[i] ? s[i] * a.scale_log2e : -INFINITY;
+      sv4[i] = ok[i] ? __builtin_fmaf(s[i], a.scale_log2e, -slope_l2e * static_cast<float>(pos - key)) : -INFINITY;
       mx = fmaxf(mx, sv4[i]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -509,7 +513,8 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
                                     const int32_t* slots, const int32_t* token_rows,
                                     const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T, int nh,
                                     int nkv, int d, int page_size, int num_pages, float scale,
-                                    int window, int nsplit, kvc_stream stream) {
+                                    int window, const float* slopes, int chunk, int nsplit,
+                                    kvc_stream stream) {
   if (!kvc_decode_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_decode_attention: unsupported shape (bfloat16, head size a multiple of 32 "
                     "up to 256, at most 16 query heads per kv head, page size a multiple of 16)");
@@ -549,8 +554,11 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
   args.num_pages = num_pages;
   args.scale_log2e = scale * kLog2e;
   args.window = window;
+  args.slopes = slopes;
+  args.chunk = chunk;
   args.nsplit = nsplit;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  kvc_note_variant(kVariantDecodeAttention, nsplit > 1 ? "decode_attention_kernel with splits" : "decode_attention_kernel");
   switch (d) {
     case 32: return launch_decode<32>(args, T, s);
     case 64: return launch_decode<64>(args, T, s);

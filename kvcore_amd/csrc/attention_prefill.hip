@@ -84,7 +84,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int single,
+    const float* __restrict__ slopes, int chunk, float* __restrict__ part_o, float* __restrict__ part_ml, int single,
     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim, int interleaved) {
   constexpr int kKeyBlocks = KB;
   constexpr int NJ = D / 16;
@@ -158,10 +158,18 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   const int n_tok = t_end - t0;
   const int pos_lo = positions[t0];
   const int pos_hi = pos_lo + n_tok - 1;  // positions rise by one along a request's tokens
-  const int first_lo = (window > 0 && pos_lo - window + 1 > 0) ? pos_lo - window + 1 : 0;
+  // the first key a token at position p sees: behind it lie the keys its window has passed and
+  // those of earlier chunks; it never falls as p rises
+  auto first_of = [&](int p) -> int {
+    int f = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    if (chunk > 0 && p >= 0 && (p / chunk) * chunk > f) f = (p / chunk) * chunk;
+    return f;
+  };
+  const int first_lo = first_of(pos_lo);
 
   // this lane's rows: column `col` of tile ct is row (wave*CT + ct)*16 + col of the block
   int my_pos[CT], my_first[CT], my_tok[CT], my_head[CT];
+  float my_slope[CT];  // in units of the raw scores: slope / scale
   bool live[CT];
   bf16x8_t qb[CT][NC];
 #pragma unroll
@@ -172,7 +180,8 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     my_tok[ct] = t0 + (live[ct] ? tq : 0);
     my_head[ct] = hk * g + rho % g;
     my_pos[ct] = live[ct] ? pos_lo + tq : -1;  // positions rise by one along a request's tokens
-    my_first[ct] = (window > 0 && my_pos[ct] - window + 1 > 0) ? my_pos[ct] - window + 1 : 0;
+    my_first[ct] = first_of(my_pos[ct]);
+    my_slope[ct] = slopes != nullptr ? slopes[my_head[ct]] * kLog2e / scale_log2e : 0.f;
     const bf16_t* qp = q + static_cast<int64_t>(my_tok[ct]) * q_stride +
                        static_cast<int64_t>(my_head[ct]) * D + 8 * quad;
 #pragma unroll
@@ -243,7 +252,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
   const bool wave_live = wave_tq_lo < n_tok;
   const int wave_pos_hi = wave_live ? pos_lo + (wave_tq_hi < n_tok ? wave_tq_hi : n_tok - 1) : -1;
   const int wave_pos_lo = wave_live ? pos_lo + wave_tq_lo : 0x7fffffff;
-  const int wave_first_hi = (wave_live && window > 0 && wave_pos_hi - window + 1 > 0) ? wave_pos_hi - window + 1 : 0;
+  const int wave_first_hi = wave_live ? first_of(wave_pos_hi) : 0;
 
   f32x4_t o_acc[CT][NJ];
   // m: the reference maximum of the raw (unscaled) scores, the same in the four lanes of a row;
@@ -483,6 +492,17 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     // every tile.  The scale is applied inside the exponent's multiply-add.
     float mx[CT];
     bool moved = false;
+    if (slopes != nullptr) {  // scalar: the distance to every key comes off its score
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const float d0 = static_cast<float>(my_pos[ct] - (kb0 * 16 + 4 * quad));
+#pragma unroll
+        for (int kbi = 0; kbi < kKeyBlocks; ++kbi)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            s[ct][kbi][i] = __builtin_fmaf(-my_slope[ct], d0 - static_cast<float>(16 * kbi + i), s[ct][kbi][i]);
+      }
+    }
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       if (!whole) {
@@ -616,7 +636,8 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                      float* part_o, float* part_ml, int nsplit, int single, const float* cos_tab,
+                      const float* slopes, int chunk, float* part_o, float* part_ml, int nsplit, int single,
+                      const float* cos_tab,
                       const float* sin_tab, int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
   const int bq = (16 * W * CT) / g;
@@ -643,8 +664,8 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   kvc_note_variant(kVariantPrefillAttention, variant);
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
-                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, part_o,
-                     part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
+                     q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, slopes, chunk,
+                     part_o, part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
   if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
@@ -654,7 +675,8 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    const bf16_t* v_cache, const int32_t* table, int table_stride,
                    const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                   float* part_o, float* part_ml, int nsplit, const float* cos_tab, const float* sin_tab,
+                   const float* slopes, int chunk, float* part_o, float* part_ml, int nsplit,
+                   const float* cos_tab, const float* sin_tab,
                    int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
   // Blocks of four waves lie two to a compute unit, blocks of eight waves one.  Tiles of 64
@@ -712,7 +734,7 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
 #define KVC_LAUNCH_PREFILL(CT_, W_)                                                                      \
   return launch_prefill_ct<D, CT_, W_>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions, \
                                        q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window, \
-                                       part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
+                                       slopes, chunk, part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
                                        interleaved, stream)
   if (waves == 8) {
     if (ct == 2) KVC_LAUNCH_PREFILL(2, 8);
@@ -738,7 +760,7 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                                      const int32_t* positions, const int32_t* q_start,
                                      const int32_t* slots, int T, int R, int nh, int nkv, int d,
                                      int page_size, int num_pages, float scale, int window,
-                                     void* part_o, void* part_ml, int nsplit, const float* cos_tab,
+                                     const float* slopes, int chunk, void* part_o, void* part_ml, int nsplit, const float* cos_tab,
                                      const float* sin_tab, int rot_dim, int interleaved,
                                      kvc_stream stream) {
   if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
@@ -768,8 +790,8 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
   if (d == 64)
     return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                               positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                              window, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                              window, slopes, chunk, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
   return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                             window, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                             window, slopes, chunk, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
 }

@@ -275,6 +275,8 @@ int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, float limit, f
 // kvc_decode_attention_max_table: the widest block table (entries per request) whose page ids
 // for one split still fit in a block's LDS; a wider one is refused, so engines check it when
 // they are built.
+// slopes (float32 [nh] or null) and chunk as for kvc_paged_attention; the kernel for portions
+// (kvc_prefill_attention) takes them too.
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_decode_attention_waves(int nh, int nkv, int d);
 int kvc_decode_attention_max_table(int nh, int nkv, int d);
@@ -284,7 +286,7 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv
                          const int32_t* slots, const int32_t* token_rows, const float* cos_tab,
                          const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T,
                          int nh, int nkv, int d, int page_size, int num_pages, float scale,
-                         int window, int nsplit, kvc_stream stream);
+                         int window, const float* slopes, int chunk, int nsplit, kvc_stream stream);
 
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds
@@ -300,7 +302,7 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
                           const void* v_cache, const int32_t* table, int table_stride,
                           const int32_t* positions, const int32_t* q_start, const int32_t* slots,
                           int T, int R, int nh, int nkv, int d, int page_size, int num_pages,
-                          float scale, int window, void* part_o, void* part_ml, int nsplit,
+                          float scale, int window, const float* slopes, int chunk, void* part_o, void* part_ml, int nsplit,
                           const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved,
                           kvc_stream stream);
 

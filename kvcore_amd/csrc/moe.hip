@@ -14,8 +14,8 @@
 //                    expert side by side in one pass, and the activation
 //                    min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + 1) on the way out.
 //                    bfloat16 operands go through the matrix cores (16 x 16 x 32, the expert's rows as
-//                    the A operand, the tokens as B) with float32 sums; float32 operands are summed
-//                    in float32 in index order.  A row's sums do not depend on which tile it is in.
+//                    the A operand, the tokens as B) with float32 sums; float32 operands, and rows
+//                    that 16-byte loads do not divide, are summed in float32 in index order.  A row's sums do not depend on which tile it is in.
 //   kvc_moe_combine  out[t] = sum_c weight[t, c] * y[t * top + c] (+ up to two more row sets),
 //                    float32, in the order of the choices.
 //   kvc_clamped_glu  the same activation for a feed-forward that every token runs.
@@ -236,11 +236,12 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   if (nf < N) store4<TO>(out + out_row * out_stride + nf, acc, N - nf);
 }
 
-// float32: a thread a (row, column) pair of the tile, sums in index order.
-template <int GATED>
-__global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
-    float* __restrict__ out, int64_t out_stride, const float* __restrict__ x, int64_t x_stride,
-    const float* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
+// Any operand type and any sizes: a thread a (row, column) pair of the tile, float32 sums in index
+// order.  The float32 path, and bfloat16 rows that 16-byte loads do not divide.
+template <int GATED, typename TI, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
+    TO* __restrict__ out, int64_t out_stride, const TI* __restrict__ x, int64_t x_stride,
+    const TI* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;
@@ -249,17 +250,18 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
   if (li >= nr) return;
   const int pair = sorted[r0 + li];
   const int64_t in_row = in_div > 0 ? pair / in_div : r0 + li;
-  const float* xr = x + in_row * x_stride;
+  const TI* xr = x + in_row * x_stride;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
   const int64_t out_row = out_sorted ? r0 + li : pair;
   for (int n = blockIdx.y * 64 + col; n < N && n < (blockIdx.y + 1) * 64; n += 16) {
-    const float* wr = w + (static_cast<int64_t>(e) * rows_per_expert + n) * K;
+    const TI* wr = w + (static_cast<int64_t>(e) * rows_per_expert + n) * K;
     float acc = 0.f, acc2 = 0.f;
     for (int k = 0; k < K; ++k) {
-      acc = fmaf(xr[k], wr[k], acc);
-      if (GATED) acc2 = fmaf(xr[k], wr[static_cast<int64_t>(N) * K + k], acc2);
+      const float xv = to_float(xr[k]);
+      acc = fmaf(xv, to_float(wr[k]), acc);
+      if (GATED) acc2 = fmaf(xv, to_float(wr[static_cast<int64_t>(N) * K + k]), acc2);
     }
-    out[out_row * out_stride + n] = GATED ? clamped_glu(acc, acc2, limit, alpha) : acc;
+    out[out_row * out_stride + n] = from_float<TO>(GATED ? clamped_glu(acc, acc2, limit, alpha) : acc);
   }
 }
 
@@ -327,40 +329,33 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
   const dim3 grid(max_tiles, (N + 63) / 64);
   if (grid.y > 65535u) return kvc_fail("kvc_moe_gemm: too many columns");
 #define KVC_MOE_ARGS sorted, tiles, num_tiles, N, K, in_div, out_sorted, limit, alpha
+#define KVC_MOE_LAUNCH(KERNEL, TI, TO)                                                                          \
+  hipLaunchKernelGGL(KERNEL, grid, dim3(256), 0, S(stream), static_cast<TO*>(out), out_stride,                   \
+                     static_cast<const TI*>(x), x_stride, static_cast<const TI*>(w), KVC_MOE_ARGS)
+  if (out_dtype != 0 && out_dtype != 1) return kvc_fail("kvc_moe_gemm: unknown dtype code");
   if (dtype == 1) {
-    if (K % 8 || x_stride % 8 || (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(w) & 15))
-      return kvc_fail("kvc_moe_gemm: bfloat16 rows must be multiples of 8 values, 16-byte aligned");
-    const bf16_t* xb = static_cast<const bf16_t*>(x);
-    const bf16_t* wb = static_cast<const bf16_t*>(w);
-    if (gated && out_dtype == 1) {
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<1, bf16_t>), grid, dim3(256), 0, S(stream), static_cast<bf16_t*>(out),
-                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
-    } else if (gated && out_dtype == 0) {
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<1, float>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
-                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
-    } else if (out_dtype == 1) {
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<0, bf16_t>), grid, dim3(256), 0, S(stream), static_cast<bf16_t*>(out),
-                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
-    } else if (out_dtype == 0) {
-      hipLaunchKernelGGL((moe_gemm_bf16_kernel<0, float>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
-                         out_stride, xb, x_stride, wb, KVC_MOE_ARGS);
+    // the matrix cores read 16 bytes at a time: rows of a multiple of 8 values, 16-byte aligned
+    const bool vectors = K % 8 == 0 && x_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+    if (vectors) {
+      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, bf16_t>), bf16_t, bf16_t);
+      else if (gated) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, float>), bf16_t, float);
+      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, bf16_t>), bf16_t, bf16_t);
+      else KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, float>), bf16_t, float);
     } else {
-      return kvc_fail("kvc_moe_gemm: unknown dtype code");
+      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, bf16_t, bf16_t>), bf16_t, bf16_t);
+      else if (gated) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, bf16_t, float>), bf16_t, float);
+      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<0, bf16_t, bf16_t>), bf16_t, bf16_t);
+      else KVC_MOE_LAUNCH((moe_gemm_plain_kernel<0, bf16_t, float>), bf16_t, float);
     }
   } else if (dtype == 0) {
     if (out_dtype != 0) return kvc_fail("kvc_moe_gemm: float32 operands give float32 rows");
-    if (gated) {
-      hipLaunchKernelGGL((moe_gemm_f32_kernel<1>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
-                         out_stride, static_cast<const float*>(x), x_stride, static_cast<const float*>(w),
-                         KVC_MOE_ARGS);
-    } else {
-      hipLaunchKernelGGL((moe_gemm_f32_kernel<0>), grid, dim3(256), 0, S(stream), static_cast<float*>(out),
-                         out_stride, static_cast<const float*>(x), x_stride, static_cast<const float*>(w),
-                         KVC_MOE_ARGS);
-    }
+    if (gated) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, float, float>), float, float);
+    else KVC_MOE_LAUNCH((moe_gemm_plain_kernel<0, float, float>), float, float);
   } else {
     return kvc_fail("kvc_moe_gemm: unknown dtype code");
   }
+#undef KVC_MOE_LAUNCH
 #undef KVC_MOE_ARGS
   return kvc_check_launch("kvc_moe_gemm");
 }

@@ -70,11 +70,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "kvc_gated_group_rmsnorm": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
-                                 F, I, I, P],
+                                 F, I, P, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_max_table": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
-        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, P, I,
+        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, P, I,
                                   P, P, I, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_mid_slices": [I, I],
@@ -421,11 +421,20 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor,
         int(write_kv), _code(qkv, "qkv"), _stream()), "kvc_qk_norm_rope_kv_write")
 
 
+def _slopes(slopes: torch.Tensor | None, nh: int) -> int | None:
+    """Pointer to the distance slopes (float32, a value per query head) of the attention kernels."""
+    if slopes is None:
+        return None
+    if slopes.shape != (nh,):
+        raise KernelError("attention: a distance slope per query head")
+    return _dev(slopes, "slopes", torch.float32)
+
+
 def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
     return bool(load().kvc_decode_attention_supported(nh, nkv, d, page_size, DTYPE_CODE.get(dtype, -1)))
 
 
-KERNEL_FAMILIES = {"prefill_attention": 0, "rope_kv_write": 1}
+KERNEL_FAMILIES = {"prefill_attention": 0, "rope_kv_write": 1, "decode_attention": 2}
 
 
 def last_variant(family: str) -> str:
@@ -504,7 +513,8 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
                      nsplit: int = 1, part_o: torch.Tensor | None = None,
                      part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
-                     write_kv: bool = False, token_rows: torch.Tensor | None = None) -> None:
+                     write_kv: bool = False, token_rows: torch.Tensor | None = None,
+                     slopes: torch.Tensor | None = None, chunk: int = 0) -> None:
     """bfloat16 attention of single tokens on the matrix cores (see the C header), with the
     rotation of each token's query and key and the write of its key and value into the cache
     (``write_kv``) in the same kernel; ``qkv`` is not changed.  With ``rot_dim = 0`` and
@@ -543,7 +553,7 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
         None if token_rows is None else _dev(token_rows, "token_rows", torch.int32),
         c, s_, int(rot_dim), int(bool(interleaved)),
         int(bool(write_kv)), T, nh, nkv, d, page_size, num_pages, float(scale),
-        int(window), int(nsplit), _stream()), "kvc_decode_attention")
+        int(window), _slopes(slopes, nh), int(chunk), int(nsplit), _stream()), "kvc_decode_attention")
 
 
 def prefill_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
@@ -555,7 +565,8 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       slots: torch.Tensor, num_reqs: int, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, nsplit: int = 1, part_o: torch.Tensor | None = None,
                       part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
-                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False) -> None:
+                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
+                      slopes: torch.Tensor | None = None, chunk: int = 0) -> None:
     """bfloat16 attention of portions of prompts on the matrix cores (see the C header).
     ``nsplit > 1`` deals every tile's keys to that many blocks; ``part_o`` (float32,
     ``T*nh*nsplit*d`` values) and ``part_ml`` (``T*nh*nsplit*2``) are then the workspace.
@@ -587,8 +598,8 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         out.data_ptr(), q.data_ptr(), q.stride(0), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
-        nh, nkv, d, page_size, num_pages, float(scale), int(window), po, pml, int(nsplit),
-        cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
+        nh, nkv, d, page_size, num_pages, float(scale), int(window), _slopes(slopes, nh), int(chunk),
+        po, pml, int(nsplit), cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
         "kvc_prefill_attention")
 
 

@@ -291,11 +291,11 @@ class PagedAttention(Mixer):
                       slots=ctx.slots, nh=self.num_heads, nkv=self.num_kv_heads, d=self.head_dim,
                       scale=self.scale, window=self.window)
         x_dtype = qkv.dtype
-        if self._slopes is not None or self.chunk > 0:
-            # scores with a distance bias or a chunked view: the general kernel
-            ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_plane_dim, slopes=self._slopes,
-                                chunk=self.chunk, **common)
-        elif not self._same_sizes():
+        # a distance bias and a chunked view are options of every attention kernel
+        common.update(slopes=self._slopes, chunk=self.chunk)
+        # a token never sees more keys than its window or its chunk holds: what the launch plans count
+        reach = min((n for n in (self.window, self.chunk) if n > 0), default=0)
+        if not self._same_sizes():
             ops.paged_attention(attn, qkv, k_cache, v_cache, dv=self.v_plane_dim, **common)
         elif ctx.max_query_len == 1 and ops.decode_attention_supported(
                 self.num_heads, self.num_kv_heads, self.head_dim, group.page_size, x_dtype):
@@ -303,7 +303,7 @@ class PagedAttention(Mixer):
             # cores, a block per (token, kv head, split)
             T = ctx.num_tokens
             waves = ops.decode_attention_waves(self.num_heads, self.num_kv_heads, self.head_dim)
-            nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len, waves, self.window)
+            nsplit = decode_splits(T, self.num_kv_heads, ctx.max_seq_len, waves, reach)
             part_o = part_ml = None
             if nsplit > 1:
                 # tokens x splits is at most the blocks wanted per kv head plus the tokens: room
@@ -335,7 +335,7 @@ class PagedAttention(Mixer):
                 # block, and several blocks per tile where few rows meet many keys
                 T = ctx.num_tokens
                 nsplit = prefill_splits(T, self.num_kv_heads, self.num_heads // self.num_kv_heads,
-                                        ctx.max_query_len, ctx.max_seq_len, self.window, ctx.num_reqs)
+                                        ctx.max_query_len, ctx.max_seq_len, reach, ctx.num_reqs)
                 part_o = part_ml = None
                 if nsplit > 1:
                     # asked for at their largest at once: a buffer that grows drops the graphs
@@ -349,6 +349,7 @@ class PagedAttention(Mixer):
                                       positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
                                       num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
                                       d=self.head_dim, scale=self.scale, window=self.window,
+                                      slopes=self._slopes, chunk=self.chunk,
                                       nsplit=nsplit, part_o=part_o, part_ml=part_ml,
                                       **(dict(cos=cos, sin=sin, rot_dim=rot_dim, interleaved=interleaved)
                                          if rotates else {}))

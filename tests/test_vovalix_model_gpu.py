@@ -29,24 +29,25 @@ def models(tmp_path_factory):
 
 
 _oracle: dict = {}
-_close_calls: dict = {}
-CLOSE_CALL = 0.04  # of the router logits' spread
+_margins: dict = {}
+CLOSE_CALL = 0.15  # of the router logits' spread
 
 
 def oracle(name, cfg, weights, tokens):
-    """The plain model's logits; it also notes at which positions a router's choice was a close
-    call (``close_calls``)."""
+    """The plain model's logits; it also notes how clear the routers' choices were at every
+    position (``routing_margin``)."""
     key = (name, tuple(tokens))
     if key not in _oracle:
         margins: list = []
         _oracle[key] = plain.vovalix_forward(cfg, weights, tokens, margins=margins)
-        worst = torch.stack(margins).min(dim=0).values if margins else torch.full((len(tokens),), float("inf"))
-        _close_calls[id(_oracle[key])] = {i for i in range(len(tokens)) if float(worst[i]) < CLOSE_CALL}
+        _margins[id(_oracle[key])] = (torch.stack(margins).min(dim=0).values if margins
+                                      else torch.full((len(tokens),), float("inf")))
     return _oracle[key]
 
 
-def close_calls(logits) -> set:
-    return _close_calls.get(id(logits), set())
+def routing_margin(logits, pos) -> float:
+    m = _margins.get(id(logits))
+    return float("inf") if m is None else float(m[pos])
 
 
 def session_for(folder, dtype, page, max_tokens, **kw):
@@ -58,32 +59,33 @@ def session_for(folder, dtype, page, max_tokens, **kw):
 def compare(got, expect_by_id, dtype):
     """Logit rows against the plain model's: the difference with its mean taken off, root mean
     square over the vocabulary, relative to the root mean square of the row itself.  float32
-    differs by the order of its sums only; bfloat16 rounds activations to 8 bits at a dozen
-    places a layer.  A router that the rounding of its input can turn (the plain model's two
-    candidates lie within ``CLOSE_CALL`` of the logits' spread) sends the token through another
-    expert, which is no error of the engine: in bfloat16 such a position is checked for finite
-    values only (float32 compares every position, so the routing itself is pinned there), and
-    since its neighbours read its keys and states, one position in fifty may reach one and a half
-    times the limit."""
+    differs by the order of its sums only, and every position must agree (which pins the routing
+    itself).  bfloat16 rounds activations to 8 bits at a dozen places a layer, and that can turn a
+    router whose two candidates lie close: the token then runs another expert, which is no error
+    of the engine.  So in bfloat16 a position may differ by more than the limit only where the
+    plain model's own routing was a close call (within ``CLOSE_CALL`` of the logits' spread), at
+    most one position in ten; and since the neighbours of such a position read its keys and
+    states, one position in fifty may reach one and a half times the limit."""
     limit = 2e-4 if dtype == torch.float32 else 6e-2
     assert got, "nothing was compared"
-    worst, compared, over = 0.0, 0, 0
+    worst, excused, over = 0.0, 0, 0
     for (rid, pos), row in sorted(got.items()):
         ref = expect_by_id[rid][pos]
         assert torch.isfinite(row).all(), f"non-finite logits at {rid}:{pos}"
-        if dtype == torch.bfloat16 and pos in close_calls(expect_by_id[rid]):
-            continue
-        compared += 1
         d = row - ref
         d = d - d.mean()
         err = float(d.pow(2).mean().sqrt() / (ref - ref.mean()).pow(2).mean().sqrt())
-        worst = max(worst, err)
-        if dtype == torch.bfloat16 and limit < err <= 1.5 * limit:
+        if err <= limit:
+            worst = max(worst, err)
+        elif dtype == torch.bfloat16 and routing_margin(expect_by_id[rid], pos) < CLOSE_CALL:
+            excused += 1
+        elif dtype == torch.bfloat16 and err <= 1.5 * limit:
             over += 1
-            continue
-        assert err <= limit, f"{rid}:{pos} differs by {err:.3e} of its size (limit {limit})"
-    assert over <= max(compared // 50, 0), f"{over} of {compared} positions lie above the limit"
-    assert compared * 2 >= len(got), "most positions must be compared"
+        else:
+            raise AssertionError(f"{rid}:{pos} differs by {err:.3e} of its size (limit {limit}; routing margin "
+                                 f"{routing_margin(expect_by_id[rid], pos):.3f})")
+    assert excused * 10 <= len(got) + 9, f"{excused} of {len(got)} positions differ by a turned router"
+    assert over * 50 <= len(got) + 49, f"{over} of {len(got)} positions lie above the limit"
     return worst
 
 

@@ -184,9 +184,11 @@ def test_small_kernels_around_the_recurrences():
 
 
 # ------------------------------------------------------------------------- attention
-def paged(q, k, v, page, *, scale, slopes, chunk, dtype, positions=None, shuffle=True):
+def paged(q, k, v, page, *, scale, slopes, chunk, dtype, positions=None, shuffle=True, kernel="general"):
     """Attention of ``q [T, H, d]`` (tokens at ``positions``, default 0..T-1) over keys and values
-    ``k, v [S, G, d / dv]`` laid into pages in a shuffled order, through the general kernel."""
+    ``k, v [S, G, d / dv]`` laid into pages in a shuffled order, through the general kernel, or
+    (bfloat16) the matrix-core kernel for portions (``"portion"``) or for single tokens
+    (``"single"``, one launch a token)."""
     from kvcore_amd.ops import library as ops
 
     S, G, d = k.shape
@@ -205,6 +207,25 @@ def paged(q, k, v, page, *, scale, slopes, chunk, dtype, positions=None, shuffle
         v_cache[pid, :, :, :n] = gpu(v[p * page:p * page + n].permute(1, 2, 0), dtype)
     pos = list(range(T)) if positions is None else positions
     out = torch.empty(T, H * dv, dtype=dtype, device=DEV)
+    slope_t = None if slopes is None else gpu(torch.tensor(slopes))
+    if kernel == "portion":
+        assert ops.prefill_attention_supported(H, G, d, page, dtype) and dv == d
+        ops.prefill_attention(out, gpu(q.reshape(T, -1), dtype), k_cache, v_cache, table=table,
+                              positions=torch.tensor(pos, dtype=torch.int32, device=DEV),
+                              q_start=torch.tensor([0, T], dtype=torch.int32, device=DEV),
+                              slots=torch.tensor([1], dtype=torch.int32, device=DEV), num_reqs=1, nh=H, nkv=G, d=d,
+                              scale=scale, slopes=slope_t, chunk=chunk)
+        assert ops.last_variant("prefill_attention").startswith("prefill_attention_kernel")
+        return out.double().cpu().view(T, H, dv)
+    if kernel == "single":
+        assert ops.decode_attention_supported(H, G, d, page, dtype) and dv == d
+        for i in range(T):
+            ops.decode_attention(out[i:i + 1], gpu(q[i:i + 1].reshape(1, -1), dtype), k_cache, v_cache, table=table,
+                                 positions=torch.tensor(pos[i:i + 1], dtype=torch.int32, device=DEV),
+                                 token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
+                                 slots=torch.tensor([1], dtype=torch.int32, device=DEV), nh=H, nkv=G, d=d,
+                                 scale=scale, slopes=slope_t, chunk=chunk)
+        return out.double().cpu().view(T, H, dv)
     ops.paged_attention(out, gpu(q.reshape(T, -1), dtype), k_cache, v_cache, table=table,
                         positions=torch.tensor(pos, dtype=torch.int32, device=DEV),
                         token_req=torch.zeros(T, dtype=torch.int32, device=DEV),
@@ -268,6 +289,42 @@ def test_a_key_that_stands_out_at_a_chunk_s_edges_and_far_back(single):
                     dtype=torch.float32, positions=pos)
         assert rel(got[-1], want[query]) < 1e-5, (chunk, marked, query)
         assert torch.allclose(got[-1, 1], v[marked, 0], atol=1e-3) == visible, (chunk, marked, query)
+
+
+@pytest.mark.parametrize("kernel", ["portion", "single"])
+@pytest.mark.parametrize("H,G,d,chunk", [(8, 2, 64, 48), (4, 4, 128, 0), (8, 1, 64, 200), (16, 2, 64, 1)])
+def test_matrix_core_kernels_with_bias_and_chunks(kernel, H, G, d, chunk):
+    """The bfloat16 kernels for portions and for single tokens against the plain function on the
+    same rounded values: every position of a prompt of 300 tokens (chunks that are no multiple of
+    the kernels' tiles of 16 and 64 keys, a chunk of one position, no chunk), then the key that
+    stands out at a chunk's edges."""
+    gen = torch.Generator().manual_seed(H + d + chunk)
+    T, page = 300, 16
+    q = normalised(torch.randn(T, H, d, generator=gen, dtype=torch.float64)).to(torch.bfloat16).double()
+    k = normalised(torch.randn(T, G, d, generator=gen, dtype=torch.float64)).to(torch.bfloat16).double()
+    v = torch.randn(T, G, d, generator=gen, dtype=torch.float64).to(torch.bfloat16).double()
+    # the plain function norms again: take that out by its own factor (the rounded rows' mean squares are not 1)
+    want = plain.chunked_distance_attention(q * q.pow(2).mean(-1, keepdim=True).sqrt(),
+                                            k * k.pow(2).mean(-1, keepdim=True).sqrt(), v, 0.3, chunk or None, 0.0)
+    rows = list(range(T)) if kernel == "portion" else [0, 1, 15, 16, 47, 48, 95, 96, 143, 144, 199, 200, 255, 256, 299]
+    got = paged(q[rows] if kernel == "single" else q, k, v, page, scale=0.3, slopes=plain.distance_slopes(H),
+                chunk=chunk, dtype=torch.bfloat16, positions=rows, kernel=kernel)
+    assert rel(got, want[rows]) < 1e-2
+    for size, marked, query in ((48, 95, 96), (48, 96, 143), (48, 96, 144), (48, 48, 95), (200, 0, 199), (200, 15, 199),
+                                (200, 199, 200), (0, 3, 299)):
+        k2 = (torch.randn(T, G, d, generator=gen, dtype=torch.float64) * 0.3)
+        k2[:, :, 0] = 0.0
+        k2[marked] = 0.0
+        k2[marked, :, 0] = 1.0
+        q2 = torch.randn(T, H, d, generator=gen, dtype=torch.float64) * 0.3
+        q2[:, :, 0] = 60.0
+        q2, k2 = normalised(q2).to(torch.bfloat16).double(), normalised(k2).to(torch.bfloat16).double()
+        visible = marked <= query and (size == 0 or marked // size == query // size)
+        rows = [query - 2, query - 1, query] if kernel == "portion" else [query]
+        got = paged(q2[rows], k2, v, page, scale=1.0, slopes=plain.distance_slopes(H), chunk=size,
+                    dtype=torch.bfloat16, positions=rows, kernel=kernel)
+        # the last head's slope is 2^-8: the marked key wins even from 300 tokens away
+        assert torch.allclose(got[-1, H - 1], v[marked, G - 1], atol=2e-2) == visible, (size, marked, query)
 
 
 # --------------------------------------------------------------------- routed experts
