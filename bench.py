@@ -20,7 +20,8 @@ Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 r
 with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
 first token of one N-token prompt in portions of 2,048), ``--sweep`` (decode at further
 batch sizes and context lengths, a line each with its share of the memory bandwidth);
-``--model 1b|70b`` and ``--batch`` change the shape.  ``--dirulorn s|m`` times the Dirulorn
+``--model 1b|70b`` and ``--batch`` change the shape.  ``--vovalix s|m`` times the Vovalix
+decoder beside the Dirulorn of equal size.  ``--dirulorn s|m`` times the Dirulorn
 decoder (state-space layers beside attention-with-recurrence layers) at layer sizes of a real
 model, prefill and decode, next to a Llama of the same width, depth, feed-forward and head
 counts, a line each.
@@ -90,10 +91,53 @@ DIRULORN_SHAPES = {
 }
 
 
+def _vovalix_layers(n, width, heads, kv, experts, top, ff, groups, keep, chunk):
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}},
+           "shared": {"ff": ff, "limit": 7.0}}
+    attention = {"type": "attention", "mlp": moe,
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125,
+                           "mask": {"size": chunk}}}
+    gla = {"type": "gla", "mlp": moe,
+           "mixer": {"heads": heads // 2, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 16}}
+    delta = {"type": "delta", "mlp": moe,
+             "mixer": {"heads": heads // 2, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "conv": 4}}
+    return [(attention, gla, delta, gla)[i % 4] for i in range(n)]
+
+
+# Vovalix at the layer sizes of a real model: of every four layers one chunked attention (keys and
+# values of 64, chunks of 1,024 positions), two gated linear attention (keys of 64, values of 128)
+# and one gated delta rule (keys and values of 128, four taps), each beside routed experts whose
+# four chosen ones and the shared one together are as wide as the dense feed-forward of the
+# Dirulorn and the Llama of the same width and depth
+VOVALIX_SHAPES = {
+    "s": {"architecture": "Vovalix", "vocab": 32000, "width": 1024, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+          "layers": _vovalix_layers(8, 1024, 16, 4, 16, 4, 1024, 4, 2, 1024)},
+    "m": {"architecture": "Vovalix", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+          "layers": _vovalix_layers(16, 2048, 32, 8, 32, 4, 2048, 8, 4, 1024)},
+}
+
+
+def bench_vovalix(args) -> int:
+    """The workloads of ``bench_dirulorn`` for a Vovalix shape beside the Dirulorn of the same
+    width and depth (the closest model the engine has: recurrent layers beside attention)."""
+    shapes = (VOVALIX_SHAPES[args.vovalix], DIRULORN_SHAPES[args.vovalix][0])
+    names = (f"vovalix-{args.vovalix}", f"dirulorn-of-vovalix-{args.vovalix}")
+    which = {"both": (0, 1), "vovalix": (0,), "dirulorn": (1,)}[args.vovalix_only]
+    return _bench_design(args, shapes, names, which, args.vovalix_workload)
+
+
 def bench_dirulorn(args) -> int:
     """Prefill (one 2,048-token prompt in one step) and decode (batch 8 and 64 from 512-token
     prompts) of a Dirulorn shape and of the Llama of equal size, through the whole engine; a
     JSON line per model and workload."""
+    shapes = DIRULORN_SHAPES[args.dirulorn]
+    names = (f"dirulorn-{args.dirulorn}", f"llama-of-dirulorn-{args.dirulorn}")
+    which = {"both": (0, 1), "dirulorn": (0,), "llama": (1,)}[args.dirulorn_only]
+    return _bench_design(args, shapes, names, which, args.dirulorn_workload)
+
+
+def _bench_design(args, shapes, names, which, workload) -> int:
     import torch
 
     from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig,
@@ -104,12 +148,10 @@ def bench_dirulorn(args) -> int:
     device = "cuda:0"
     torch.cuda.set_device(0)
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
-    shapes = DIRULORN_SHAPES[args.dirulorn]
-    which = {"both": (0, 1), "dirulorn": (0,), "llama": (1,)}[args.dirulorn_only]
     for index in which:
         cfg = shapes[index]
-        name = f"dirulorn-{args.dirulorn}" if index == 0 else f"llama-of-dirulorn-{args.dirulorn}"
-        vocab = cfg["vocab"] if index == 0 else cfg["vocab_size"]
+        name = names[index]
+        vocab = cfg["vocab"] if "vocab" in cfg else cfg["vocab_size"]
         model = build_model(".", dtype, device, load_format="random", seed=0, config_override=cfg)
         seqs = 64
         pages = seqs * -(-(PREFILL_TOKENS + 512 + 256) // args.page_size) + 1
@@ -129,7 +171,7 @@ def bench_dirulorn(args) -> int:
                                prompt_token_ids=[rng.randrange(vocab) for _ in range(n_prompt)])
 
         times = []
-        for _ in range(4 if args.dirulorn_workload in ("all", "prefill") else 0):
+        for _ in range(4 if workload in ("all", "prefill") else 0):
             new_request(PREFILL_TOKENS, 1)
             torch.cuda.synchronize()
             t_start = time.perf_counter()
@@ -145,7 +187,7 @@ def bench_dirulorn(args) -> int:
                               "ms": round(sec * 1e3, 3), "tokens_per_s": round(PREFILL_TOKENS / sec, 1),
                               "param_gib": round(params / 2**30, 3)}), flush=True)
         for batch in (8, 64):
-            if args.dirulorn_workload not in ("all", f"decode{batch}"):
+            if workload not in ("all", f"decode{batch}"):
                 continue
             steps, warmup = args.steps, min(args.warmup, 8)
             for _ in range(batch):
@@ -209,6 +251,13 @@ def parse_args():
                    help="with --dirulorn: run one of the two models only (for profiling)")
     p.add_argument("--dirulorn-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
                    help="with --dirulorn: run one of the workloads only (for profiling)")
+    p.add_argument("--vovalix", default=None, choices=sorted(VOVALIX_SHAPES),
+                   help="instead of the contract's line: prefill and decode of a Vovalix shape beside the "
+                        "Dirulorn of the same width and depth; a line per model and workload")
+    p.add_argument("--vovalix-only", default="both", choices=["both", "vovalix", "dirulorn"],
+                   help="with --vovalix: run one of the two models only (for profiling)")
+    p.add_argument("--vovalix-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
+                   help="with --vovalix: run one of the workloads only (for profiling)")
     p.add_argument("--sweep", action="store_true",
                    help="instead of the default run: decode at batch 1..64 and at contexts of 8k, 32k "
                         "and 128k tokens, a line each")
@@ -361,6 +410,8 @@ def main() -> int:
         return 2
     if args.dirulorn:
         return bench_dirulorn(args)
+    if args.vovalix:
+        return bench_vovalix(args)
     import torch
 
     from kvcore_amd import (CacheConfig, DeviceConfig, KVCoreConfig, LoadConfig, ModelConfig,

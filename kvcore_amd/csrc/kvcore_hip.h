@@ -242,12 +242,19 @@ int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* 
 // sorted[i].  dtype is that of x and w.
 int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
                   int groups, int keep, kvc_stream stream);
-int kvc_moe_max_tiles(int pairs, int E);
+// Tiles hold up to tile_rows rows, 16 or 64 (kvc_moe_tile_rows says which a step's size asks
+// for; 64 is for bfloat16 with K a multiple of 32).
+int kvc_moe_tile_rows(int pairs, int E);
+// The router's logits (x [T, H] of x_dtype times router [E, H] float32, float32 sums in index order)
+// and the choice of kvc_moe_route in one kernel.
+int kvc_moe_router(int32_t* choice, float* weight, const void* x, int64_t x_stride, int x_dtype,
+                   const float* router, int T, int H, int E, int top, int groups, int keep, kvc_stream stream);
+int kvc_moe_max_tiles(int pairs, int E, int tile_rows);
 int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int32_t* choice,
-                  int pairs, int E, int max_tiles, kvc_stream stream);
+                  int pairs, int E, int max_tiles, int tile_rows, kvc_stream stream);
 int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                  const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
-                 const int32_t* num_tiles, int max_tiles, int N, int K, int in_div, int out_sorted,
+                 const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div, int out_sorted,
                  int gated, float limit, float alpha, kvc_stream stream);
 // out[t] = sum_c weight[t, c] * y[t * top + c] + add0[t] + add1[t] (either may be null; add0 of
 // dtype add0_dtype, add1 float32), float32.

@@ -6,7 +6,7 @@
 //   delta rule  S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T   (g_t, beta_t scalars)
 // and in both o_t = S^T (q_scale q_t), read after the token's write.  A block owns one (request, head, tile
 // of VT value channels); the NSL threads that share a column of the state are neighbouring lanes
-// (their partial sums meet through lane shuffles, in one fixed order) and each keeps NPT rows in
+// (their partial sums meet through lane permutations, in one fixed order) and each keeps NPT rows in
 // registers; q, k, the factors and v of 16 tokens at a time go through LDS.  A request whose
 // first token of the step is at position 0 starts from zero, any other from its slot's state;
 // the state goes back to the slot at the end.  What a token's result is depends on its request's
@@ -32,14 +32,34 @@ __device__ __forceinline__ float softplus_ff(float x) { return fmaxf(x, 0.f) + l
 // log(sigmoid(x)) = -softplus(-x)
 __device__ __forceinline__ float log_sigmoid_f(float x) { return -softplus_ff(-x); }
 
-template <int NPT, int DELTA>
+// The sum of a value over the NSL (4 or 16) neighbouring lanes that share a column, by lane
+// permutations inside a row of 16 lanes (no trip through LDS): neighbours in a quad, the quads of a
+// half row, the two halves.  Every lane of the group ends with the same bits.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int NSL>
+__device__ __forceinline__ float group_sum(float v) {
+  static_assert(NSL == 4 || NSL == 16, "columns are shared by 4 or by 16 lanes");
+  v += dpp_f<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+  v += dpp_f<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+  if (NSL == 16) {
+    v += dpp_f<0x141>(v);  // row_half_mirror
+    v += dpp_f<0x140>(v);  // row_mirror
+  }
+  return v;
+}
+
+template <int NPT, int DELTA, int NSL>
 __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ decay,
     int64_t decay_stride, const float* __restrict__ beta, int64_t beta_stride, float* __restrict__ state,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int nqk, int d,
-    int dv, int VT, int NSL, float q_scale) {
+    int dv, float q_scale) {
+  constexpr int VT = 256 / NSL;  // value channels a block
   extern __shared__ float lds[];
   float* q_s = lds;               // [LSC][d]
   float* k_s = q_s + LSC * d;     // [LSC][d]
@@ -97,37 +117,53 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       float acc = 0.f;
       if (DELTA) {
         const float g = a_s[2 * tt], bt = a_s[2 * tt + 1];
-        float kd = 0.f;
+        float kd0 = 0.f, kd1 = 0.f;  // two running sums: half as long a chain of dependent operations
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
+        for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
           if (n < d) {
             s[i] *= g;
-            kd = fmaf(s[i], kt[n], kd);
+            kd0 = fmaf(s[i], kt[n], kd0);
+          }
+          if (n + NSL < d) {
+            s[i + 1] *= g;
+            kd1 = fmaf(s[i + 1], kt[n + NSL], kd1);
           }
         }
-        for (int o = 1; o < NSL; o <<= 1) kd += __shfl_xor(kd, o, kWave);
+        const float kd = group_sum<NSL>(kd0 + kd1);
         const float u = bt * (vv - kd);
+        float acc1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
+        for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
           if (n < d) {
             s[i] = fmaf(kt[n], u, s[i]);
             acc = fmaf(s[i], qt[n], acc);
           }
+          if (n + NSL < d) {
+            s[i + 1] = fmaf(kt[n + NSL], u, s[i + 1]);
+            acc1 = fmaf(s[i + 1], qt[n + NSL], acc1);
+          }
         }
+        acc += acc1;
       } else {
         const float* at = a_s + tt * d;
+        float acc1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) {
+        for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
           if (n < d) {
             s[i] = fmaf(at[n], s[i], kt[n] * vv);
             acc = fmaf(s[i], qt[n], acc);
           }
+          if (n + NSL < d) {
+            s[i + 1] = fmaf(at[n + NSL], s[i + 1], kt[n + NSL] * vv);
+            acc1 = fmaf(s[i + 1], qt[n + NSL], acc1);
+          }
         }
+        acc += acc1;
       }
-      for (int o = 1; o < NSL; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+      acc = group_sum<NSL>(acc);
       if (ns == 0 && c_ok) out[static_cast<int64_t>(t0 + tt) * width + h * dv + c] = acc;
     }
   }
@@ -218,30 +254,34 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   if (R == 0) return 0;
   // tiles of 64 value channels with 4 threads a column, or, where that leaves compute units
   // without a block, tiles of 16 with 16 threads a column
-  int VT = 64, NSL = 4;
   const int64_t wide_blocks = static_cast<int64_t>(R) * nh * ((dv + 63) / 64);
-  if (dv < 64 || wide_blocks < kvc_device_compute_units()) {
-    VT = 16;
-    NSL = 16;
-  }
+  const bool narrow = dv < 64 || wide_blocks < kvc_device_compute_units();
+  const int NSL = narrow ? 16 : 4, VT = 256 / NSL;
   const dim3 grid(R, nh, (dv + VT - 1) / VT);
   if (grid.y > 65535u || grid.z > 65535u) return kvc_fail("kvc_linear_state_scan: grid too large");
-  const dim3 block(VT * NSL);
   const size_t lds = sizeof(float) * (2 * LSC * d + LSC * (delta_rule ? 2 : d) + LSC * VT);
   const int per_thread = (d + NSL - 1) / NSL;
-#define KVC_LSCAN(NPT, DELTA)                                                                           \
-  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA>), grid, block, lds, S(stream), out, q, q_stride, \
-                     k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state, positions, \
-                     token_req, q_start, slots, nh, nqk, d, dv, VT, NSL, q_scale)
-#define KVC_LSCAN_N(NPT)        \
-  do {                          \
-    if (delta_rule) {           \
-      KVC_LSCAN(NPT, 1);        \
-    } else {                    \
-      KVC_LSCAN(NPT, 0);        \
-    }                           \
+#define KVC_LSCAN(NPT, DELTA, NSL_)                                                                          \
+  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_>), grid, dim3(256), lds, S(stream), out, q,    \
+                     q_stride, k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state,       \
+                     positions, token_req, q_start, slots, nh, nqk, d, dv, q_scale)
+#define KVC_LSCAN_N(NPT)                 \
+  do {                                   \
+    if (delta_rule && narrow) {          \
+      KVC_LSCAN(NPT, 1, 16);             \
+    } else if (delta_rule) {             \
+      KVC_LSCAN(NPT, 1, 4);              \
+    } else if (narrow) {                 \
+      KVC_LSCAN(NPT, 0, 16);             \
+    } else {                             \
+      KVC_LSCAN(NPT, 0, 4);              \
+    }                                    \
   } while (0)
-  if (per_thread <= 8) {
+  if (per_thread <= 2) {
+    KVC_LSCAN_N(2);
+  } else if (per_thread <= 4) {
+    KVC_LSCAN_N(4);
+  } else if (per_thread <= 8) {
     KVC_LSCAN_N(8);
   } else if (per_thread <= 16) {
     KVC_LSCAN_N(16);

@@ -8,8 +8,10 @@
 //   kvc_moe_route    scores = softmax(logits) in float32; the `keep` groups whose best score is
 //                    highest; the `top` best experts of those groups (the lower index on a tie);
 //                    weights = chosen scores / (their sum + 1e-20).  A wave a token.
+//   kvc_moe_router   the router's product (float32 sums in index order over rows of either dtype) and
+//                    the choice in one kernel.
 //   kvc_moe_align    pairs sorted by expert: sorted[i] = pair index (token * top + choice), and a
-//                    list of tiles of up to 16 sorted rows that belong to one expert each.
+//                    list of tiles of up to 16 (or 64) sorted rows that belong to one expert each.
 //   kvc_moe_gemm     for every tile, rows x that expert's matrix.  Gated: gate and up rows of the
 //                    expert side by side in one pass, and the activation
 //                    min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + 1) on the way out.
@@ -33,6 +35,7 @@ namespace {
 #define S(stream) reinterpret_cast<hipStream_t>(stream)
 
 constexpr int kTileRows = 16;
+constexpr int kBigTileRows = 64;
 
 __device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
   g = fminf(g, limit);
@@ -53,16 +56,10 @@ __device__ __forceinline__ void wave_argmax(float& val, int& idx) {
   }
 }
 
-__global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
-                                                        const float* __restrict__ logits, int T, int E,
-                                                        int top, int groups, int keep) {
-  extern __shared__ float lds[];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  float* sc = lds + wave * (E + groups);  // scores, then the groups' best
-  float* gs = sc + E;
-  const int t = blockIdx.x * 4 + wave;
-  if (t >= T) return;  // the whole wave
-  const float* z = logits + static_cast<int64_t>(t) * E;
+// One token's choice by one wave: z [E] logits (global or LDS), sc [E] and gs [groups] LDS scratch
+// (sc may be z itself).
+__device__ __forceinline__ void route_one(int32_t* __restrict__ choice, float* __restrict__ weight, const float* z,
+                                          float* sc, float* gs, int lane, int E, int top, int groups, int keep) {
   float mx = -INFINITY;
   for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
   mx = wave_max(mx);
@@ -129,8 +126,75 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ ch
   }
   const float norm = 1.f / (total + 1e-20f);
   if (lane < top) {
-    choice[static_cast<int64_t>(t) * top + lane] = mine_idx;
-    weight[static_cast<int64_t>(t) * top + lane] = mine * norm;
+    choice[lane] = mine_idx;
+    weight[lane] = mine * norm;
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
+                                                        const float* __restrict__ logits, int T, int E,
+                                                        int top, int groups, int keep) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  float* sc = lds + wave * (E + groups);  // scores, then the groups' best
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;  // the whole wave
+  route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top,
+            logits + static_cast<int64_t>(t) * E, sc, sc + E, lane, E, top, groups, keep);
+}
+
+// The router whole: logits = x W^T in float32 (x of either dtype, its values as they are; every
+// logit one running sum in index order, so that it does not depend on the batch), then the choice
+// as in moe_route_kernel.  A block takes TB tokens; the rows' and the router's chunks of 128 values
+// along K go through LDS; thread (token, eg) sums the experts eg, eg + 256 / TB, ...
+template <typename T, int TB>
+__global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
+                                                         const T* __restrict__ x, int64_t x_stride,
+                                                         const float* __restrict__ wr, int T_, int H, int E, int top,
+                                                         int groups, int keep) {
+  constexpr int KC = 128, KP = KC + 1, EG = 256 / TB, EMAX = 64 / EG;  // 64 experts a pass
+  extern __shared__ float lds[];
+  float* x_s = lds;                  // [TB][KP]
+  float* w_s = x_s + TB * KP;        // [EG * EMAX][KP]
+  float* z_s = w_s + EG * EMAX * KP; // [TB][E + groups]: logits, then scores and the groups' best
+  const int tok = threadIdx.x / EG, eg = threadIdx.x % EG;
+  const int t0 = blockIdx.x * TB;
+  for (int e0 = 0; e0 < E; e0 += EG * EMAX) {
+    float acc[EMAX];
+#pragma unroll
+    for (int j = 0; j < EMAX; ++j) acc[j] = 0.f;
+    const int ne = (E - e0 < EG * EMAX) ? E - e0 : EG * EMAX;
+    for (int k0 = 0; k0 < H; k0 += KC) {
+      const int nk = (H - k0 < KC) ? H - k0 : KC;
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < TB * KC; idx += 256) {
+        const int r = idx / KC, k = idx - r * KC;
+        x_s[r * KP + k] = (t0 + r < T_ && k < nk) ? to_float(x[static_cast<int64_t>(t0 + r) * x_stride + k0 + k]) : 0.f;
+      }
+      for (int idx = threadIdx.x; idx < ne * KC; idx += 256) {
+        const int r = idx / KC, k = idx - r * KC;
+        w_s[r * KP + k] = k < nk ? wr[static_cast<int64_t>(e0 + r) * H + k0 + k] : 0.f;
+      }
+      __syncthreads();
+      for (int k = 0; k < nk; ++k) {
+        const float xv = x_s[tok * KP + k];
+#pragma unroll
+        for (int j = 0; j < EMAX; ++j)
+          if (eg + EG * j < ne) acc[j] = fmaf(xv, w_s[(eg + EG * j) * KP + k], acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < EMAX; ++j)
+      if (eg + EG * j < ne) z_s[tok * (E + groups) + e0 + eg + EG * j] = acc[j];
+  }
+  __syncthreads();
+  // a wave a token from here on
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  for (int r = wave; r < TB; r += 4) {
+    const int t = t0 + r;
+    if (t >= T_) continue;  // the whole wave
+    route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top, z_s + r * (E + groups),
+              z_s + r * (E + groups), z_s + r * (E + groups) + E, lane, E, top, groups, keep);
   }
 }
 
@@ -138,7 +202,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ ch
 __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ sorted, int32_t* __restrict__ tiles,
                                                          int32_t* __restrict__ num_tiles,
                                                          const int32_t* __restrict__ choice, int pairs, int E,
-                                                         int max_tiles) {
+                                                         int max_tiles, int tile_rows) {
   extern __shared__ int32_t ilds[];
   int32_t* count = ilds;           // [E]
   int32_t* offset = count + E;     // [E + 1]
@@ -155,10 +219,10 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
     for (int e = 0; e < E; ++e) {
       offset[e] = at;
       cursor[e] = 0;
-      for (int r = 0; r < count[e] && nt < max_tiles; r += kTileRows, ++nt) {
+      for (int r = 0; r < count[e] && nt < max_tiles; r += tile_rows, ++nt) {
         tiles[3 * nt] = e;
         tiles[3 * nt + 1] = at + r;
-        tiles[3 * nt + 2] = (count[e] - r < kTileRows) ? count[e] - r : kTileRows;
+        tiles[3 * nt + 2] = (count[e] - r < tile_rows) ? count[e] - r : tile_rows;
       }
       at += count[e];
     }
@@ -176,7 +240,12 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
   }
 }
 
-// bfloat16: a block of four waves takes one tile of rows and 64 columns (16 a wave).
+// bfloat16: a block of four waves takes one tile of rows and 64 columns (16 a wave).  A round covers
+// 64 values along K: lane (li, lk) fetches the 16 values from 16 lk of its weight row and of its
+// token row (32 contiguous bytes, so that the four lanes of a row read one 128-byte line) and the two
+// matrix instructions of the round take its first and its second eight (both operands are dealt the
+// same way, so each product still sums over all of K); the next round's values are asked for
+// before this round's products.
 template <int GATED, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
@@ -189,41 +258,58 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int n0 = (blockIdx.y * 4 + wave) * 16;
   if (n0 >= N) return;
   const int li = lane & 15, lk = lane >> 4;
-  // B operand: token row li of the tile, 8 values of k from 8 * lk
+  // B operand: token row li of the tile; A operand: the expert's row n0 + li
   const bool row_ok = li < nr;
   const int pair = row_ok ? sorted[r0 + li] : 0;
   const int64_t in_row = in_div > 0 ? pair / in_div : r0 + li;
-  const bf16_t* xr = x + in_row * x_stride + 8 * lk;
-  // A operand: the expert's row n0 + li
+  const bf16_t* xr = x + in_row * x_stride + 16 * lk;
   const int wrow = n0 + li < N ? n0 + li : N - 1;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
-  const bf16_t* wr = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 8 * lk;
+  const bf16_t* wr = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 16 * lk;
   const bf16_t* wr2 = wr + static_cast<int64_t>(N) * K;  // the up rows follow the gate rows
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-  const int k_main = K & ~31;
-  for (int k = 0; k < k_main; k += 32) {
-    bf16x8_t b = zero8();
-    if (row_ok) b = *reinterpret_cast<const bf16x8_t*>(xr + k);
-    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(wr + k);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-    if (GATED) {
-      const bf16x8_t a2 = *reinterpret_cast<const bf16x8_t*>(wr2 + k);
-      acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc2, 0, 0, 0);
+  const int k_main = K & ~63;
+  bf16x8_t an[2], a2n[2], bn[2];
+  auto fetch = [&](int k) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      an[h] = *reinterpret_cast<const bf16x8_t*>(wr + k + 8 * h);
+      if (GATED) a2n[h] = *reinterpret_cast<const bf16x8_t*>(wr2 + k + 8 * h);
+      bn[h] = row_ok ? *reinterpret_cast<const bf16x8_t*>(xr + k + 8 * h) : zero8();
+    }
+  };
+  if (k_main > 0) fetch(0);
+  for (int k = 0; k < k_main; k += 64) {
+    bf16x8_t a[2], a2[2], b[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      a[h] = an[h];
+      if (GATED) a2[h] = a2n[h];
+      b[h] = bn[h];
+    }
+    if (k + 64 < k_main) fetch(k + 64);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], b[h], acc, 0, 0, 0);
+      if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[h], b[h], acc2, 0, 0, 0);
     }
   }
-  if (k_main < K) {  // a ragged end along K: element by element, zeros beyond
-    bf16x8_t a = zero8(), a2 = zero8(), b = zero8();
-    for (int i = 0; i < 8; ++i) {
-      const int kk = k_main + 8 * lk + i;
-      if (kk < K) {
-        const __bf16* wp = reinterpret_cast<const __bf16*>(wr + k_main);
-        a[i] = wp[i];
-        if (GATED) a2[i] = reinterpret_cast<const __bf16*>(wr2 + k_main)[i];
-        if (row_ok) b[i] = reinterpret_cast<const __bf16*>(xr + k_main)[i];
+  if (k_main < K) {  // a ragged end along K (a multiple of 8): element by element, zeros beyond
+    bf16x8_t a[2], a2[2], b[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      a[h] = zero8(); a2[h] = zero8(); b[h] = zero8();
+      for (int i = 0; i < 8; ++i) {
+        const int off = k_main + 8 * h + i;  // from the lane's own start 16 lk
+        if (off + 16 * lk < K) {
+          a[h][i] = reinterpret_cast<const __bf16*>(wr)[off];
+          if (GATED) a2[h][i] = reinterpret_cast<const __bf16*>(wr2)[off];
+          if (row_ok) b[h][i] = reinterpret_cast<const __bf16*>(xr)[off];
+        }
       }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], b[h], acc, 0, 0, 0);
+      if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[h], b[h], acc2, 0, 0, 0);
     }
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-    if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b, acc2, 0, 0, 0);
   }
   // lane holds column (token) li, rows (features) n0 + 4 * lk + i
   if (!row_ok) return;
@@ -234,6 +320,105 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int64_t out_row = out_sorted ? r0 + li : pair;
   const int nf = n0 + 4 * lk;
   if (nf < N) store4<TO>(out + out_row * out_stride + nf, acc, N - nf);
+}
+
+// bfloat16, tiles of 64 rows: a block of four waves takes the tile's rows and 128 columns (gated;
+// 256 otherwise).  The rows' chunk of 32 values along K goes through LDS, which all waves read as
+// the B operand (four row blocks of 16); every wave fetches the weight rows of its own columns
+// straight into registers as the A operand (NF blocks of 16 columns, for gate and for up), one
+// chunk ahead of the products.  Every fetched weight meets 64 rows, every row 128 or 256 columns.
+template <int GATED, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
+    TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
+    const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+  constexpr int NF = GATED ? 2 : 4;   // column blocks of 16 a wave
+  constexpr int NR = kBigTileRows / 16;
+  constexpr int KROW = 40;            // a row's 32 values in LDS, padded against bank conflicts
+  __shared__ __attribute__((aligned(16))) bf16_t x_s[kBigTileRows * KROW];
+  const int tile = blockIdx.x;
+  if (tile >= *num_tiles) return;
+  const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int li = lane & 15, lk = lane >> 4;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * NF;
+  const bool wave_live = n0 < N;  // the same for the whole wave
+  // staging: thread t brings 8 values of row t / 4 of the tile
+  const int srow = threadIdx.x >> 2, spart = threadIdx.x & 3;
+  const bool srow_ok = srow < nr;
+  int64_t in_row = 0;
+  if (srow_ok) in_row = in_div > 0 ? sorted[r0 + srow] / in_div : r0 + srow;
+  const bf16_t* xp = x + in_row * x_stride + 8 * spart;
+  const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* wp[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int wrow = n0 + 16 * f + li < N ? n0 + 16 * f + li : N - 1;
+    wp[f] = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 8 * lk;
+  }
+  const int64_t up_off = static_cast<int64_t>(N) * K;
+  f32x4_t acc[NF][NR], acc2[GATED ? NF : 1][NR];
+#pragma unroll
+  for (int f = 0; f < NF; ++f)
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      acc[f][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (GATED) acc2[f][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  uint4 x_next = uint4{0u, 0u, 0u, 0u};
+  bf16x8_t w_next[NF], w2_next[GATED ? NF : 1];
+  auto fetch = [&](int k) {
+    if (srow_ok) x_next = *reinterpret_cast<const uint4*>(xp + k);
+    if (wave_live) {
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        w_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + k);
+        if (GATED) w2_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + up_off + k);
+      }
+    }
+  };
+  fetch(0);
+  for (int k = 0; k < K; k += 32) {
+    __syncthreads();  // the chunk before has been read by every wave
+    *reinterpret_cast<uint4*>(x_s + srow * KROW + 8 * spart) = x_next;
+    bf16x8_t wa[NF], wa2[GATED ? NF : 1];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      wa[f] = w_next[f];
+      if (GATED) wa2[f] = w2_next[f];
+    }
+    if (k + 32 < K) fetch(k + 32);
+    __syncthreads();
+    if (wave_live) {  // scalar: matrix instructions are skipped by a branch, never by a lane mask
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(x_s + (16 * r + li) * KROW + 8 * lk);
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          acc[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[f], b, acc[f][r], 0, 0, 0);
+          if (GATED) acc2[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa2[f], b, acc2[f][r], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!wave_live) return;
+  // lane holds row 16 r + li of the tile, columns n0 + 16 f + 4 lk + i
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int row = 16 * r + li;
+    if (row >= nr) continue;
+    const int64_t out_row = out_sorted ? r0 + row : sorted[r0 + row];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      f32x4_t v = acc[f][r];
+      if (GATED) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = clamped_glu(v[i], acc2[f][r][i], limit, alpha);
+      }
+      const int nf = n0 + 16 * f + 4 * lk;
+      if (nf < N) store4<TO>(out + out_row * out_stride + nf, v, N - nf);
+    }
+  }
 }
 
 // Any operand type and any sizes: a thread a (row, column) pair of the tile, float32 sums in index
@@ -306,27 +491,68 @@ extern "C" int kvc_moe_route(int32_t* choice, float* weight, const float* logits
   return kvc_check_launch("kvc_moe_route");
 }
 
-extern "C" int kvc_moe_max_tiles(int pairs, int E) { return (pairs + kTileRows - 1) / kTileRows + E; }
+extern "C" int kvc_moe_router(int32_t* choice, float* weight, const void* x, int64_t x_stride, int x_dtype,
+                              const float* router, int T, int H, int E, int top, int groups, int keep,
+                              kvc_stream stream) {
+  if (T < 0 || H <= 0 || E <= 0 || top <= 0 || top > E || top > kWave || groups <= 0 || E % groups || keep <= 0 ||
+      keep > groups || x_stride < H)
+    return kvc_fail("kvc_moe_router: bad sizes (at most 64 choices; the experts in equal groups)");
+  if (T == 0) return 0;
+  // blocks of 16 tokens where those fill the chip, else of 4
+  const bool big = T >= 16 * kvc_device_compute_units() / 4;
+  const int TB = big ? 16 : 4;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(TB) * 129 + static_cast<size_t>(64) * 129 +
+                                      static_cast<size_t>(TB) * (E + groups));
+  if (lds > 160 * 1024) return kvc_fail("kvc_moe_router: too many experts for a block's LDS");
+  const dim3 grid((T + TB - 1) / TB);
+#define KVC_ROUTER(Tp, TB_)                                                                                     \
+  do {                                                                                                          \
+    if (lds > 64 * 1024) {                                                                                      \
+      const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<Tp, TB_>),   \
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+      if (attr != hipSuccess) return kvc_fail("kvc_moe_router: the kernel's LDS size was refused");            \
+    }                                                                                                           \
+    hipLaunchKernelGGL((moe_router_kernel<Tp, TB_>), grid, dim3(256), lds, S(stream), choice, weight,           \
+                       static_cast<const Tp*>(x), x_stride, router, T, H, E, top, groups, keep);                \
+  } while (0)
+  if (x_dtype == 1 && big) KVC_ROUTER(bf16_t, 16);
+  else if (x_dtype == 1) KVC_ROUTER(bf16_t, 4);
+  else if (x_dtype == 0 && big) KVC_ROUTER(float, 16);
+  else if (x_dtype == 0) KVC_ROUTER(float, 4);
+  else return kvc_fail("kvc_moe_router: unknown dtype code");
+#undef KVC_ROUTER
+  return kvc_check_launch("kvc_moe_router");
+}
+
+extern "C" int kvc_moe_max_tiles(int pairs, int E, int tile_rows) {
+  return (pairs + tile_rows - 1) / tile_rows + E;
+}
+
+// Tiles of 64 rows where the experts have that many rows on average (portions of prompts): the
+// tiled kernel then uses every fetched weight four times as often; tiles of 16 otherwise.
+extern "C" int kvc_moe_tile_rows(int pairs, int E) { return pairs >= 64 * E ? kBigTileRows : kTileRows; }
 
 extern "C" int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int32_t* choice,
-                             int pairs, int E, int max_tiles, kvc_stream stream) {
-  if (pairs < 0 || E <= 0 || max_tiles < kvc_moe_max_tiles(pairs, E))
+                             int pairs, int E, int max_tiles, int tile_rows, kvc_stream stream) {
+  if (tile_rows != kTileRows && tile_rows != kBigTileRows) return kvc_fail("kvc_moe_align: tiles of 16 or 64 rows");
+  if (pairs < 0 || E <= 0 || max_tiles < kvc_moe_max_tiles(pairs, E, tile_rows))
     return kvc_fail("kvc_moe_align: bad sizes, or room for fewer tiles than the routing may need");
   const size_t lds = sizeof(int32_t) * (3 * E + 1);
   if (lds > 60000) return kvc_fail("kvc_moe_align: too many experts");
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), lds, S(stream), sorted, tiles, num_tiles, choice,
-                     pairs, E, max_tiles);
+                     pairs, E, max_tiles, tile_rows);
   return kvc_check_launch("kvc_moe_align");
 }
 
 extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                             const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
-                            const int32_t* num_tiles, int max_tiles, int N, int K, int in_div,
+                            const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div,
                             int out_sorted, int gated, float limit, float alpha, kvc_stream stream) {
   if (max_tiles < 0 || N <= 0 || K <= 0 || x_stride < K || out_stride < N)
     return kvc_fail("kvc_moe_gemm: bad sizes");
+  if (tile_rows != kTileRows && tile_rows != kBigTileRows) return kvc_fail("kvc_moe_gemm: tiles of 16 or 64 rows");
   if (max_tiles == 0) return 0;
-  const dim3 grid(max_tiles, (N + 63) / 64);
+  dim3 grid(max_tiles, (N + 63) / 64);
   if (grid.y > 65535u) return kvc_fail("kvc_moe_gemm: too many columns");
 #define KVC_MOE_ARGS sorted, tiles, num_tiles, N, K, in_div, out_sorted, limit, alpha
 #define KVC_MOE_LAUNCH(KERNEL, TI, TO)                                                                          \
@@ -337,7 +563,14 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
     // the matrix cores read 16 bytes at a time: rows of a multiple of 8 values, 16-byte aligned
     const bool vectors = K % 8 == 0 && x_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(w) & 15) == 0;
-    if (vectors) {
+    if (tile_rows == kBigTileRows) {
+      if (!vectors || K % 32) return kvc_fail("kvc_moe_gemm: tiles of 64 rows need K to be a multiple of 32");
+      grid.y = gated ? (N + 127) / 128 : (N + 255) / 256;
+      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, bf16_t>), bf16_t, bf16_t);
+      else if (gated) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, float>), bf16_t, float);
+      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, bf16_t>), bf16_t, bf16_t);
+      else KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, float>), bf16_t, float);
+    } else if (vectors) {
       if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, bf16_t>), bf16_t, bf16_t);
       else if (gated) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, float>), bf16_t, float);
       else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, bf16_t>), bf16_t, bf16_t);
@@ -350,6 +583,7 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
     }
   } else if (dtype == 0) {
     if (out_dtype != 0) return kvc_fail("kvc_moe_gemm: float32 operands give float32 rows");
+    if (tile_rows != kTileRows) return kvc_fail("kvc_moe_gemm: float32 operands take tiles of 16 rows");
     if (gated) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, float, float>), float, float);
     else KVC_MOE_LAUNCH((moe_gemm_plain_kernel<0, float, float>), float, float);
   } else {

@@ -54,9 +54,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_unit_heads": [P, L, I, I, I, F, F, P],
         "kvc_head_rmsnorm_gate": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_moe_route": [P, P, P, I, I, I, I, I, P],
-        "kvc_moe_max_tiles": [I, I],
-        "kvc_moe_align": [P, P, P, P, I, I, I, P],
-        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, F, F, P],
+        "kvc_moe_router": [P, P, P, L, I, P, I, I, I, I, I, I, P],
+        "kvc_moe_max_tiles": [I, I, I],
+        "kvc_moe_tile_rows": [I, I],
+        "kvc_moe_align": [P, P, P, P, I, I, I, I, P],
+        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, P],
         "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, P],
         "kvc_clamped_glu": [P, P, I, I, F, F, I, P],
         "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
@@ -1333,24 +1335,47 @@ def moe_route(choice: torch.Tensor, weight: torch.Tensor, logits: torch.Tensor, 
            "kvc_moe_route")
 
 
-def moe_max_tiles(pairs: int, experts: int) -> int:
-    return int(load().kvc_moe_max_tiles(pairs, experts))
+def moe_router(choice: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, router: torch.Tensor, *, top: int,
+               groups: int = 1, keep: int = 1) -> None:
+    """``moe_route`` of the logits ``x @ router.T`` (float32 sums in index order; ``x [T, H]`` of
+    either dtype, ``router [E, H]`` float32) without storing the logits."""
+    T, H = x.shape
+    E = router.shape[0]
+    if router.shape != (E, H) or choice.shape != (T, top) or weight.shape != (T, top) or x.stride(1) != 1:
+        raise KernelError("moe_router: shapes do not match")
+    _check(load().kvc_moe_router(_dev(choice, "choice", torch.int32), _dev(weight, "weight", torch.float32),
+                                 x.data_ptr(), x.stride(0), _code(x, "x"), _dev(router, "router", torch.float32),
+                                 T, H, E, top, groups, keep, _stream()), "kvc_moe_router")
+
+
+def moe_tile_rows(pairs: int, experts: int, x: torch.Tensor | None = None, k_sizes: tuple[int, ...] = ()) -> int:
+    """Rows a tile of the experts' products holds for a step of this size: 64 where the experts
+    have that many rows on average and the operands allow (bfloat16, every K a multiple of 32), else 16."""
+    rows = int(load().kvc_moe_tile_rows(pairs, experts))
+    if rows > 16 and (x is None or x.dtype != torch.bfloat16 or any(k % 32 for k in k_sizes)):
+        return 16
+    return rows
+
+
+def moe_max_tiles(pairs: int, experts: int, tile_rows: int = 16) -> int:
+    return int(load().kvc_moe_max_tiles(pairs, experts, tile_rows))
 
 
 def moe_align(sorted_pairs: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, choice: torch.Tensor,
-              experts: int) -> None:
-    """(token, choice) pairs sorted by expert, and the list of row tiles (``tiles [>= max_tiles, 3]``)."""
+              experts: int, tile_rows: int = 16) -> None:
+    """(token, choice) pairs sorted by expert, and the list of row tiles (``tiles [>= max_tiles, 3]``)
+    of up to ``tile_rows`` rows."""
     pairs = choice.numel()
     if sorted_pairs.numel() < pairs or tiles.dim() != 2 or tiles.shape[1] != 3 or num_tiles.numel() < 1:
         raise KernelError("moe_align: buffers too small")
     _check(load().kvc_moe_align(_dev(sorted_pairs, "sorted", torch.int32), _dev(tiles, "tiles", torch.int32),
                                 _dev(num_tiles, "num_tiles", torch.int32), _dev(choice, "choice", torch.int32),
-                                pairs, experts, tiles.shape[0], _stream()), "kvc_moe_align")
+                                pairs, experts, tiles.shape[0], tile_rows, _stream()), "kvc_moe_align")
 
 
 def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tiles: torch.Tensor,
              num_tiles: torch.Tensor, *, pairs: int, experts: int, in_div: int, out_sorted: bool, gated: bool,
-             limit: float = 0.0, alpha: float = 0.0) -> None:
+             limit: float = 0.0, alpha: float = 0.0, tile_rows: int = 16) -> None:
     """Every expert's product over its own rows.  ``w`` is ``[experts * N, K]`` (``experts * 2N``
     rows when ``gated``: each expert's gate rows, then its up rows); ``out [pairs, N]``."""
     N = out.shape[1]
@@ -1358,11 +1383,11 @@ def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: 
     rows = experts * N * (2 if gated else 1)
     if w.shape != (rows, K) or out.shape[0] < pairs or x.dtype != w.dtype or out.stride(1) != 1 or x.stride(1) != 1:
         raise KernelError("moe_gemm: shapes do not match")
-    max_tiles = min(tiles.shape[0], moe_max_tiles(pairs, experts))
+    max_tiles = min(tiles.shape[0], moe_max_tiles(pairs, experts, tile_rows))
     _check(load().kvc_moe_gemm(out.data_ptr(), out.stride(0), _code(out, "out"), x.data_ptr(), x.stride(0),
                                _dev(w, "w"), _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
                                _dev(tiles, "tiles", torch.int32), _dev(num_tiles, "num_tiles", torch.int32),
-                               max_tiles, N, K, int(in_div), int(bool(out_sorted)), int(bool(gated)),
+                               max_tiles, tile_rows, N, K, int(in_div), int(bool(out_sorted)), int(bool(gated)),
                                float(limit), float(alpha), _stream()), "kvc_moe_gemm")
 
 

@@ -74,30 +74,25 @@ class RoutedExperts(FeedForward):
         p, H, E, I, top = self.params, self.hidden_size, self.experts, self.expert_size, self.top
         T = ctx.num_tokens
         pairs = T * top
-        # the router reads the rows in float32 (of bfloat16 rows, their values as they are)
-        if x.dtype == torch.float32:
-            xf = x
-        else:
-            xf = ctx.buf(f"moe_x_f32:{H}", H, torch.float32)
-            ops.to_float(xf, x)
-        logits = ctx.buf(f"moe_logits:{E}", E, torch.float32)
-        ops.gemm_f32(logits, xf, p["router.weight"], None)
+        # the router reads the rows as they are and sums in float32; logits and choice in one kernel
         choice = ctx.buf(f"moe_choice:{top}", top, torch.int32)
         weight = ctx.buf(f"moe_weight:{top}", top, torch.float32)
-        ops.moe_route(choice, weight, logits, top=top, groups=self.groups, keep=self.keep)
+        ops.moe_router(choice, weight, x, p["router.weight"], top=top, groups=self.groups, keep=self.keep)
         cap = ctx.buffers.token_capacity
         sorted_pairs = ctx.buffers.get(f"moe_sorted:{top}", pairs, 1, torch.int32, reserve=cap * top).view(-1)
-        max_tiles = ops.moe_max_tiles(pairs, E)
+        # portions of prompts give the experts rows enough for tiles of 64, single tokens tiles of 16
+        tile_rows = ops.moe_tile_rows(pairs, E, x, (H, I))
+        max_tiles = ops.moe_max_tiles(pairs, E, tile_rows)
         tiles = ctx.buffers.get(f"moe_tiles:{top}:{E}", max_tiles, 3, torch.int32,
-                                reserve=ops.moe_max_tiles(cap * top, E))
+                                reserve=ops.moe_max_tiles(cap * top, E, 16))
         num_tiles = ctx.buffers.get("moe_num_tiles", 1, 1, torch.int32).view(-1)
-        ops.moe_align(sorted_pairs, tiles, num_tiles, choice, E)
+        ops.moe_align(sorted_pairs, tiles, num_tiles, choice, E, tile_rows)
         act = ctx.buffers.get(f"moe_act:{I}", pairs, I, ctx.dtype, reserve=cap * top)
         ops.moe_gemm(act, x, p["experts.gate_up"], sorted_pairs, tiles, num_tiles, pairs=pairs, experts=E,
-                     in_div=top, out_sorted=True, gated=True, limit=self.limit, alpha=self.alpha)
+                     in_div=top, out_sorted=True, gated=True, limit=self.limit, alpha=self.alpha, tile_rows=tile_rows)
         y = ctx.buffers.get(f"moe_y:{H}", pairs, H, torch.float32, reserve=cap * top)
         ops.moe_gemm(y, act, p["experts.down"], sorted_pairs, tiles, num_tiles, pairs=pairs, experts=E,
-                     in_div=0, out_sorted=False, gated=False)
+                     in_div=0, out_sorted=False, gated=False, tile_rows=tile_rows)
         shared = None
         if self.shared_size:
             S = self.shared_size

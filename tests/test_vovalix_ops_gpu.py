@@ -351,6 +351,40 @@ def test_routing_against_the_plain_rule(E, top, groups, keep):
         assert float(weight[t, live:].abs().sum()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("E,top,groups,keep,H,T", [(6, 2, 3, 2, 96, 75), (32, 4, 8, 4, 256, 1100), (2, 2, 2, 2, 40, 1),
+                                                   (70, 6, 10, 3, 130, 9), (130, 3, 1, 1, 64, 20)])
+def test_router_product_and_choice_in_one_kernel(dtype, E, top, groups, keep, H, T):
+    """The fused router against the plain rule on the same rows; the logits are float32 sums of the
+    rows as they are, the same for a token alone and among a thousand (blocks of 4 and of 16 tokens)."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(E + T)
+    x = torch.randn(T, H, generator=gen, dtype=torch.float64)
+    x = x.to(dtype).double()
+    w = (torch.randn(E, H, generator=gen, dtype=torch.float64) * 0.5).float().double()
+    choice = torch.empty(T, top, dtype=torch.int32, device=DEV)
+    weight = torch.empty(T, top, dtype=torch.float32, device=DEV)
+    ops.moe_router(choice, weight, gpu(x, dtype), gpu(w), top=top, groups=groups, keep=keep)
+    logits = x @ w.T
+    scores = torch.softmax(logits, dim=-1)
+    checked = 0
+    for t in range(T):
+        if plain.route_margin(logits[t], top, groups, keep) < 1e-4:
+            continue  # a tie within float32's reach
+        want_e, want_w = plain.route(scores[t], top, groups, keep)
+        assert choice[t].tolist() == want_e, t
+        assert torch.allclose(weight[t].double().cpu(), want_w, atol=1e-5), t
+        checked += 1
+    assert checked >= T * 0.9
+    # a token's result does not depend on the batch: the first rows alone give the same bits
+    n = min(T, 3)
+    c2 = torch.empty(n, top, dtype=torch.int32, device=DEV)
+    w2 = torch.empty(n, top, dtype=torch.float32, device=DEV)
+    ops.moe_router(c2, w2, gpu(x[:n], dtype), gpu(w), top=top, groups=groups, keep=keep)
+    assert torch.equal(c2, choice[:n]) and torch.equal(w2, weight[:n])
+
+
 def expert_weights(E, H, I, gen, shared=0):
     w = {"router": torch.randn(E, H, generator=gen, dtype=torch.float64) * 0.5}
     for e in range(E):
