@@ -245,7 +245,7 @@ int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, in
 // Tiles hold up to tile_rows rows, 16 or 64 (kvc_moe_tile_rows says which a step's size asks
 // for; 64 is for bfloat16 with K a multiple of 32).
 int kvc_moe_tile_rows(int pairs, int E);
-// The router's logits (x [T, H] of x_dtype times router [E, H] float32, float32 sums in index order)
+// The router's logits (x [T, H] of x_dtype times router [E, H] float32, float32 sums in one fixed order)
 // and the choice of kvc_moe_route in one kernel.
 int kvc_moe_router(int32_t* choice, float* weight, const void* x, int64_t x_stride, int x_dtype,
                    const float* router, int T, int H, int E, int top, int groups, int keep, kvc_stream stream);

@@ -51,7 +51,7 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int NPT, int DELTA, int NSL>
+template <int NPT, int DELTA, int NSL, int FULL>
 __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ decay,
@@ -60,7 +60,9 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int nqk, int d,
     int dv, float q_scale) {
   constexpr int VT = 256 / NSL;  // value channels a block
-  extern __shared__ float lds[];
+  // FULL: d == NPT * NSL, so no row needs a bound, and a thread's rows of q, k and the factors lie
+  // side by side in LDS (row n of a token at (n % NSL) * NPT + n / NSL), read 16 bytes at a time
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* q_s = lds;               // [LSC][d]
   float* k_s = q_s + LSC * d;     // [LSC][d]
   float* a_s = k_s + LSC * d;     // [LSC][d] (key decay) or [LSC][2] (delta: g, beta)
@@ -95,9 +97,10 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     for (int idx = tid; idx < nt * d; idx += nthreads) {
       const int tt = idx / d, n = idx - tt * d;
       const int64_t t = t0 + tt;
-      q_s[idx] = q[t * q_stride + hk * d + n] * q_scale;
-      k_s[idx] = k[t * k_stride + hk * d + n];
-      if (!DELTA) a_s[idx] = decay[t * decay_stride + h * d + n];
+      const int at = FULL ? tt * d + (n % NSL) * NPT + n / NSL : idx;
+      q_s[at] = q[t * q_stride + hk * d + n] * q_scale;
+      k_s[at] = k[t * k_stride + hk * d + n];
+      if (!DELTA) a_s[at] = decay[t * decay_stride + h * d + n];
     }
     if (DELTA) {
       for (int tt = tid; tt < nt; tt += nthreads) {
@@ -111,8 +114,9 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float* qt = q_s + tt * d;
-      const float* kt = k_s + tt * d;
+      const float* qt = q_s + tt * d + (FULL ? ns * NPT : ns);
+      const float* kt = k_s + tt * d + (FULL ? ns * NPT : ns);
+      constexpr int ST = FULL ? 1 : NSL;  // from one of the thread's rows to its next, in LDS
       const float vv = v_s[tt * VT + pl];
       float acc = 0.f;
       if (DELTA) {
@@ -121,13 +125,13 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 #pragma unroll
         for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
-          if (n < d) {
+          if (FULL || n < d) {
             s[i] *= g;
-            kd0 = fmaf(s[i], kt[n], kd0);
+            kd0 = fmaf(s[i], kt[ST * i], kd0);
           }
-          if (n + NSL < d) {
+          if (FULL || n + NSL < d) {
             s[i + 1] *= g;
-            kd1 = fmaf(s[i + 1], kt[n + NSL], kd1);
+            kd1 = fmaf(s[i + 1], kt[ST * (i + 1)], kd1);
           }
         }
         const float kd = group_sum<NSL>(kd0 + kd1);
@@ -136,29 +140,29 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
 #pragma unroll
         for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
-          if (n < d) {
-            s[i] = fmaf(kt[n], u, s[i]);
-            acc = fmaf(s[i], qt[n], acc);
+          if (FULL || n < d) {
+            s[i] = fmaf(kt[ST * i], u, s[i]);
+            acc = fmaf(s[i], qt[ST * i], acc);
           }
-          if (n + NSL < d) {
-            s[i + 1] = fmaf(kt[n + NSL], u, s[i + 1]);
-            acc1 = fmaf(s[i + 1], qt[n + NSL], acc1);
+          if (FULL || n + NSL < d) {
+            s[i + 1] = fmaf(kt[ST * (i + 1)], u, s[i + 1]);
+            acc1 = fmaf(s[i + 1], qt[ST * (i + 1)], acc1);
           }
         }
         acc += acc1;
       } else {
-        const float* at = a_s + tt * d;
+        const float* at = a_s + tt * d + (FULL ? ns * NPT : ns);
         float acc1 = 0.f;
 #pragma unroll
         for (int i = 0; i < NPT; i += 2) {
           const int n = ns + NSL * i;
-          if (n < d) {
-            s[i] = fmaf(at[n], s[i], kt[n] * vv);
-            acc = fmaf(s[i], qt[n], acc);
+          if (FULL || n < d) {
+            s[i] = fmaf(at[ST * i], s[i], kt[ST * i] * vv);
+            acc = fmaf(s[i], qt[ST * i], acc);
           }
-          if (n + NSL < d) {
-            s[i + 1] = fmaf(at[n + NSL], s[i + 1], kt[n + NSL] * vv);
-            acc1 = fmaf(s[i + 1], qt[n + NSL], acc1);
+          if (FULL || n + NSL < d) {
+            s[i + 1] = fmaf(at[ST * (i + 1)], s[i + 1], kt[ST * (i + 1)] * vv);
+            acc1 = fmaf(s[i + 1], qt[ST * (i + 1)], acc1);
           }
         }
         acc += acc1;
@@ -261,10 +265,18 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   if (grid.y > 65535u || grid.z > 65535u) return kvc_fail("kvc_linear_state_scan: grid too large");
   const size_t lds = sizeof(float) * (2 * LSC * d + LSC * (delta_rule ? 2 : d) + LSC * VT);
   const int per_thread = (d + NSL - 1) / NSL;
-#define KVC_LSCAN(NPT, DELTA, NSL_)                                                                          \
-  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_>), grid, dim3(256), lds, S(stream), out, q,    \
-                     q_stride, k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state,       \
+#define KVC_LSCAN_F(NPT, DELTA, NSL_, FULL_)                                                                  \
+  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_>), grid, dim3(256), lds, S(stream), out, \
+                     q, q_stride, k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state,    \
                      positions, token_req, q_start, slots, nh, nqk, d, dv, q_scale)
+#define KVC_LSCAN(NPT, DELTA, NSL_)        \
+  do {                                     \
+    if (d == NPT * NSL_) {                 \
+      KVC_LSCAN_F(NPT, DELTA, NSL_, 1);    \
+    } else {                               \
+      KVC_LSCAN_F(NPT, DELTA, NSL_, 0);    \
+    }                                      \
+  } while (0)
 #define KVC_LSCAN_N(NPT)                 \
   do {                                   \
     if (delta_rule && narrow) {          \
@@ -292,6 +304,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   }
 #undef KVC_LSCAN_N
 #undef KVC_LSCAN
+#undef KVC_LSCAN_F
   return kvc_check_launch("kvc_linear_state_scan");
 }
 

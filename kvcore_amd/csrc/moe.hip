@@ -8,8 +8,8 @@
 //   kvc_moe_route    scores = softmax(logits) in float32; the `keep` groups whose best score is
 //                    highest; the `top` best experts of those groups (the lower index on a tie);
 //                    weights = chosen scores / (their sum + 1e-20).  A wave a token.
-//   kvc_moe_router   the router's product (float32 sums in index order over rows of either dtype) and
-//                    the choice in one kernel.
+//   kvc_moe_router   the router's product (float32 sums in one fixed order over rows of either dtype)
+//                    and the choice in one kernel.
 //   kvc_moe_align    pairs sorted by expert: sorted[i] = pair index (token * top + choice), and a
 //                    list of tiles of up to 16 (or 64) sorted rows that belong to one expert each.
 //   kvc_moe_gemm     for every tile, rows x that expert's matrix.  Gated: gate and up rows of the
@@ -143,58 +143,76 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ ch
             logits + static_cast<int64_t>(t) * E, sc, sc + E, lane, E, top, groups, keep);
 }
 
-// The router whole: logits = x W^T in float32 (x of either dtype, its values as they are; every
-// logit one running sum in index order, so that it does not depend on the batch), then the choice
-// as in moe_route_kernel.  A block takes TB tokens; the rows' and the router's chunks of 128 values
-// along K go through LDS; thread (token, eg) sums the experts eg, eg + 256 / TB, ...
-template <typename T, int TB>
+// The router whole: logits = x W^T in float32 (x of either dtype, its values as they are), then the
+// choice as in moe_route_kernel.  A wave takes TOK tokens: lane l sums the products of the values
+// 4 l .. 4 l + 3 of every 256 along K for each of up to 32 experts at a time (a fetched piece of the
+// router's row meets all TOK tokens), the 64 partial sums of a logit are added in lane order through
+// LDS: one fixed order, whatever the batch.
+template <typename T, int TOK>
 __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
                                                          const T* __restrict__ x, int64_t x_stride,
                                                          const float* __restrict__ wr, int T_, int H, int E, int top,
-                                                         int groups, int keep) {
-  constexpr int KC = 128, KP = KC + 1, EG = 256 / TB, EMAX = 64 / EG;  // 64 experts a pass
+                                                         int groups, int keep, int vectors) {
+  constexpr int EB = 32, PR = EB + 1;
   extern __shared__ float lds[];
-  float* x_s = lds;                  // [TB][KP]
-  float* w_s = x_s + TB * KP;        // [EG * EMAX][KP]
-  float* z_s = w_s + EG * EMAX * KP; // [TB][E + groups]: logits, then scores and the groups' best
-  const int tok = threadIdx.x / EG, eg = threadIdx.x % EG;
-  const int t0 = blockIdx.x * TB;
-  for (int e0 = 0; e0 < E; e0 += EG * EMAX) {
-    float acc[EMAX];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  float* part = lds + wave * (kWave * PR);                               // [64][EB + 1]
+  float* z = lds + 4 * kWave * PR + wave * TOK * (E + groups);           // [TOK][E + groups]
+  const int t0 = (blockIdx.x * 4 + wave) * TOK;
+  if (t0 >= T_) return;  // the whole wave
+  for (int e0 = 0; e0 < E; e0 += EB) {
+    const int ne = (E - e0 < EB) ? E - e0 : EB;
+    float acc[TOK][EB];
 #pragma unroll
-    for (int j = 0; j < EMAX; ++j) acc[j] = 0.f;
-    const int ne = (E - e0 < EG * EMAX) ? E - e0 : EG * EMAX;
-    for (int k0 = 0; k0 < H; k0 += KC) {
-      const int nk = (H - k0 < KC) ? H - k0 : KC;
-      __syncthreads();
-      for (int idx = threadIdx.x; idx < TB * KC; idx += 256) {
-        const int r = idx / KC, k = idx - r * KC;
-        x_s[r * KP + k] = (t0 + r < T_ && k < nk) ? to_float(x[static_cast<int64_t>(t0 + r) * x_stride + k0 + k]) : 0.f;
-      }
-      for (int idx = threadIdx.x; idx < ne * KC; idx += 256) {
-        const int r = idx / KC, k = idx - r * KC;
-        w_s[r * KP + k] = k < nk ? wr[static_cast<int64_t>(e0 + r) * H + k0 + k] : 0.f;
-      }
-      __syncthreads();
-      for (int k = 0; k < nk; ++k) {
-        const float xv = x_s[tok * KP + k];
+    for (int j = 0; j < TOK; ++j)
 #pragma unroll
-        for (int j = 0; j < EMAX; ++j)
-          if (eg + EG * j < ne) acc[j] = fmaf(xv, w_s[(eg + EG * j) * KP + k], acc[j]);
+      for (int e = 0; e < EB; ++e) acc[j][e] = 0.f;
+    for (int k = 4 * lane; k < H; k += 4 * kWave) {
+      float xv[TOK][4];
+#pragma unroll
+      for (int j = 0; j < TOK; ++j) {
+        const T* xr = x + static_cast<int64_t>(t0 + j < T_ ? t0 + j : t0) * x_stride + k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xv[j][i] = (k + i < H) ? to_float(xr[i]) : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < EB; ++e) {
+        if (e < ne) {
+          const float* wp = wr + static_cast<int64_t>(e0 + e) * H + k;
+          float wv[4];
+          if (vectors) {
+            const float4 v4 = *reinterpret_cast<const float4*>(wp);
+            wv[0] = v4.x; wv[1] = v4.y; wv[2] = v4.z; wv[3] = v4.w;
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wv[i] = (k + i < H) ? wp[i] : 0.f;
+          }
+#pragma unroll
+          for (int j = 0; j < TOK; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][e] = fmaf(xv[j][i], wv[i], acc[j][e]);
+        }
       }
     }
 #pragma unroll
-    for (int j = 0; j < EMAX; ++j)
-      if (eg + EG * j < ne) z_s[tok * (E + groups) + e0 + eg + EG * j] = acc[j];
+    for (int j = 0; j < TOK; ++j) {
+#pragma unroll
+      for (int e = 0; e < EB; ++e) part[lane * PR + e] = acc[j][e];
+      __builtin_amdgcn_wave_barrier();
+      if (lane < ne) {
+        float sum = 0.f;
+        for (int l = 0; l < kWave; ++l) sum += part[l * PR + lane];
+        z[j * (E + groups) + e0 + lane] = sum;
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
-  __syncthreads();
-  // a wave a token from here on
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  for (int r = wave; r < TB; r += 4) {
-    const int t = t0 + r;
-    if (t >= T_) continue;  // the whole wave
-    route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top, z_s + r * (E + groups),
-              z_s + r * (E + groups), z_s + r * (E + groups) + E, lane, E, top, groups, keep);
+  for (int j = 0; j < TOK; ++j) {
+    const int t = t0 + j;
+    if (t >= T_) break;  // the whole wave
+    float* zr = z + j * (E + groups);
+    route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top, zr, zr, zr + E, lane, E,
+              top, groups, keep);
   }
 }
 
@@ -498,27 +516,28 @@ extern "C" int kvc_moe_router(int32_t* choice, float* weight, const void* x, int
       keep > groups || x_stride < H)
     return kvc_fail("kvc_moe_router: bad sizes (at most 64 choices; the experts in equal groups)");
   if (T == 0) return 0;
-  // blocks of 16 tokens where those fill the chip, else of 4
-  const bool big = T >= 16 * kvc_device_compute_units() / 4;
-  const int TB = big ? 16 : 4;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(TB) * 129 + static_cast<size_t>(64) * 129 +
-                                      static_cast<size_t>(TB) * (E + groups));
+  // four tokens a wave where the waves then still fill the chip, else one
+  const bool big = T >= 4 * 4 * kvc_device_compute_units();
+  const int TOK = big ? 4 : 1;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(4) * 64 * 33 + static_cast<size_t>(4) * TOK * (E + groups));
   if (lds > 160 * 1024) return kvc_fail("kvc_moe_router: too many experts for a block's LDS");
-  const dim3 grid((T + TB - 1) / TB);
-#define KVC_ROUTER(Tp, TB_)                                                                                     \
+  const dim3 grid((T + 4 * TOK - 1) / (4 * TOK));
+  // 16-byte loads of the router's rows where the rows allow
+  const int vectors = H % 4 == 0 && (reinterpret_cast<uintptr_t>(router) & 15) == 0;
+#define KVC_ROUTER(Tp, TOK_)                                                                                    \
   do {                                                                                                          \
     if (lds > 64 * 1024) {                                                                                      \
-      const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<Tp, TB_>),   \
+      const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_router_kernel<Tp, TOK_>),  \
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
       if (attr != hipSuccess) return kvc_fail("kvc_moe_router: the kernel's LDS size was refused");            \
     }                                                                                                           \
-    hipLaunchKernelGGL((moe_router_kernel<Tp, TB_>), grid, dim3(256), lds, S(stream), choice, weight,           \
-                       static_cast<const Tp*>(x), x_stride, router, T, H, E, top, groups, keep);                \
+    hipLaunchKernelGGL((moe_router_kernel<Tp, TOK_>), grid, dim3(256), lds, S(stream), choice, weight,          \
+                       static_cast<const Tp*>(x), x_stride, router, T, H, E, top, groups, keep, vectors);       \
   } while (0)
-  if (x_dtype == 1 && big) KVC_ROUTER(bf16_t, 16);
-  else if (x_dtype == 1) KVC_ROUTER(bf16_t, 4);
-  else if (x_dtype == 0 && big) KVC_ROUTER(float, 16);
-  else if (x_dtype == 0) KVC_ROUTER(float, 4);
+  if (x_dtype == 1 && big) KVC_ROUTER(bf16_t, 4);
+  else if (x_dtype == 1) KVC_ROUTER(bf16_t, 1);
+  else if (x_dtype == 0 && big) KVC_ROUTER(float, 4);
+  else if (x_dtype == 0) KVC_ROUTER(float, 1);
   else return kvc_fail("kvc_moe_router: unknown dtype code");
 #undef KVC_ROUTER
   return kvc_check_launch("kvc_moe_router");

@@ -1337,7 +1337,7 @@ def moe_route(choice: torch.Tensor, weight: torch.Tensor, logits: torch.Tensor, 
 
 def moe_router(choice: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, router: torch.Tensor, *, top: int,
                groups: int = 1, keep: int = 1) -> None:
-    """``moe_route`` of the logits ``x @ router.T`` (float32 sums in index order; ``x [T, H]`` of
+    """``moe_route`` of the logits ``x @ router.T`` (float32 sums in one fixed order; ``x [T, H]`` of
     either dtype, ``router [E, H]`` float32) without storing the logits."""
     T, H = x.shape
     E = router.shape[0]
