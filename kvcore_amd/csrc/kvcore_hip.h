@@ -207,7 +207,8 @@ int kvc_gated_group_rmsnorm(void* out, int out_dtype, const float* y, const void
                             int width, int groups, kvc_stream stream);
 
 // ---- mixers whose state is a float32 matrix S [d, dv] per head (linear_attention.hip).  The batch
-// is described as for the recurrent mixers above; state is [slots, nh, d, dv] float32.
+// is described as for the recurrent mixers above; state is [slots, nh, dpad, dv] float32, dpad = d
+// rounded up to a multiple of 4, a head's element (n, c) at ((n / 4) * dv + c) * 4 + n % 4.
 // Per head h (its q and k come from head h / (nh / nqk) of nqk heads of d), token by token:
 //   delta_rule 0:  S = diag(decay[t, h, :]) S + k v^T            (decay rows of nh * d values)
 //   delta_rule 1:  S = decay[t, h] S;  u = beta[t, h] (v - S^T k);  S = S + k u^T

@@ -9,7 +9,8 @@
 // (their partial sums meet through lane permutations, in one fixed order) and each keeps NPT rows in
 // registers; q, k, the factors and v of 16 tokens at a time go through LDS.  A request whose
 // first token of the step is at position 0 starts from zero, any other from its slot's state;
-// the state goes back to the slot at the end.  What a token's result is depends on its request's
+// the state goes back to the slot at the end (kept there with its rows in fours: element (n, c) of a
+// head at ((n / 4) * dv + c) * 4 + n % 4, the row count rounded up to a multiple of four).  What a token's result is depends on its request's
 // earlier tokens only, not on how they were cut into steps or what else the batch holds.
 
 #include <hip/hip_runtime.h>
@@ -51,7 +52,7 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int NPT, int DELTA, int NSL, int FULL>
+template <int NPT, int DELTA, int NSL, int FULL, int PF>
 __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ decay,
@@ -63,10 +64,6 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   // FULL: d == NPT * NSL, so no row needs a bound, and a thread's rows of q, k and the factors lie
   // side by side in LDS (row n of a token at (n % NSL) * NPT + n / NSL), read 16 bytes at a time
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  float* q_s = lds;               // [LSC][d]
-  float* k_s = q_s + LSC * d;     // [LSC][d]
-  float* a_s = k_s + LSC * d;     // [LSC][d] (key decay) or [LSC][2] (delta: g, beta)
-  float* v_s = a_s + LSC * (DELTA ? 2 : d);  // [LSC][VT]
   const int r = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * VT;
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int ns = tid % NSL, pl = tid / NSL;
@@ -83,36 +80,20 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     return;
   }
   const int hk = h / (nh / nqk);
-  float* st = state + (static_cast<int64_t>(slots[r]) * nh + h) * d * dv;
+  // a head's state in memory: rows in fours, [ceil(d / 4)][dv][4], so that the four lanes that share a
+  // column (and their neighbours' columns) read and write one contiguous run
+  const int dpad = (d + 3) & ~3;
+  float* st = state + (static_cast<int64_t>(slots[r]) * nh + h) * dpad * dv;
+  auto st_at = [&](int n) -> int64_t { return (static_cast<int64_t>(n >> 2) * dv + c) * 4 + (n & 3); };
   const bool fresh = positions[b] == 0;
   float s[NPT];
 #pragma unroll
   for (int i = 0; i < NPT; ++i) {
     const int n = ns + NSL * i;
-    s[i] = (!fresh && c_ok && n < d) ? st[static_cast<int64_t>(n) * dv + c] : 0.f;
+    s[i] = (!fresh && c_ok && n < d) ? st[st_at(n)] : 0.f;
   }
-  for (int t0 = b; t0 < e; t0 += LSC) {
-    const int nt = (e - t0 < LSC) ? e - t0 : LSC;
-    __syncthreads();
-    for (int idx = tid; idx < nt * d; idx += nthreads) {
-      const int tt = idx / d, n = idx - tt * d;
-      const int64_t t = t0 + tt;
-      const int at = FULL ? tt * d + (n % NSL) * NPT + n / NSL : idx;
-      q_s[at] = q[t * q_stride + hk * d + n] * q_scale;
-      k_s[at] = k[t * k_stride + hk * d + n];
-      if (!DELTA) a_s[at] = decay[t * decay_stride + h * d + n];
-    }
-    if (DELTA) {
-      for (int tt = tid; tt < nt; tt += nthreads) {
-        a_s[2 * tt] = decay[static_cast<int64_t>(t0 + tt) * decay_stride + h];
-        a_s[2 * tt + 1] = beta[static_cast<int64_t>(t0 + tt) * beta_stride + h];
-      }
-    }
-    for (int idx = tid; idx < nt * VT; idx += nthreads) {
-      const int tt = idx / VT, cc = c0 + idx - tt * VT;
-      v_s[idx] = cc < dv ? v[static_cast<int64_t>(t0 + tt) * v_stride + h * dv + cc] : 0.f;
-    }
-    __syncthreads();
+  // one stage's tokens, from the LDS buffers given
+  auto work_stage = [&](const float* q_s, const float* k_s, const float* a_s, const float* v_s, int t0, int nt) {
     for (int tt = 0; tt < nt; ++tt) {
       const float* qt = q_s + tt * d + (FULL ? ns * NPT : ns);
       const float* kt = k_s + tt * d + (FULL ? ns * NPT : ns);
@@ -170,12 +151,105 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       acc = group_sum<NSL>(acc);
       if (ns == 0 && c_ok) out[static_cast<int64_t>(t0 + tt) * width + h * dv + c] = acc;
     }
+  };
+  if constexpr (PF) {
+    // Two sets of LDS buffers: while a stage is worked on, the next stage's q, k, factors and v are on
+    // their way from memory into registers, and go into the other set afterwards (a block has one
+    // wave a SIMD and nothing else to hide that latency behind).
+    constexpr int QN = LSC * NPT * NSL / 256;  // values of q (and of k) a thread brings a stage
+    constexpr int VN = LSC * VT / 256;
+    const int set = 2 * LSC * d + LSC * (DELTA ? 2 : d) + LSC * VT;
+    float qn[QN], kn[QN], an[DELTA ? 2 : QN], vn[VN];
+    auto fetch = [&](int t0, int nt) {
+#pragma unroll
+      for (int j = 0; j < QN; ++j) {
+        const int idx = tid + 256 * j, tt = idx / d, n = idx - tt * d;
+        const int64_t t = t0 + (tt < nt ? tt : 0);
+        qn[j] = q[t * q_stride + hk * d + n] * q_scale;
+        kn[j] = k[t * k_stride + hk * d + n];
+        if (!DELTA) an[j] = decay[t * decay_stride + h * d + n];
+      }
+      if (DELTA) {
+        const int64_t t = t0 + (tid < nt ? tid : 0);
+        an[0] = decay[t * decay_stride + h];
+        an[1] = beta[t * beta_stride + h];
+      }
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const int idx = tid + 256 * j, tt = idx / VT, cc = c0 + idx - tt * VT;
+        const int64_t t = t0 + (tt < nt ? tt : 0);
+        vn[j] = cc < dv ? v[t * v_stride + h * dv + cc] : 0.f;
+      }
+    };
+    auto stash = [&](float* base) {
+      float* q_s = base;
+      float* k_s = q_s + LSC * d;
+      float* a_s = k_s + LSC * d;
+      float* v_s = a_s + LSC * (DELTA ? 2 : d);
+#pragma unroll
+      for (int j = 0; j < QN; ++j) {
+        const int idx = tid + 256 * j, tt = idx / d, n = idx - tt * d;
+        const int at = tt * d + (n % NSL) * NPT + n / NSL;
+        q_s[at] = qn[j];
+        k_s[at] = kn[j];
+        if (!DELTA) a_s[at] = an[j];
+      }
+      if (DELTA && tid < LSC) {
+        a_s[2 * tid] = an[0];
+        a_s[2 * tid + 1] = an[1];
+      }
+#pragma unroll
+      for (int j = 0; j < VN; ++j) v_s[tid + 256 * j] = vn[j];
+    };
+    fetch(b, (e - b < LSC) ? e - b : LSC);
+    stash(lds);
+    __syncthreads();
+    int which = 0;
+    for (int t0 = b; t0 < e; t0 += LSC) {
+      const int nt = (e - t0 < LSC) ? e - t0 : LSC;
+      const bool more = t0 + LSC < e;
+      if (more) fetch(t0 + LSC, (e - t0 - LSC < LSC) ? e - t0 - LSC : LSC);
+      float* base = lds + which * set;
+      work_stage(base, base + LSC * d, base + 2 * LSC * d, base + 2 * LSC * d + LSC * (DELTA ? 2 : d), t0, nt);
+      if (more) stash(lds + (which ^ 1) * set);
+      __syncthreads();
+      which ^= 1;
+    }
+  } else {
+    float* q_s = lds;               // [LSC][d]
+    float* k_s = q_s + LSC * d;     // [LSC][d]
+    float* a_s = k_s + LSC * d;     // [LSC][d] (key decay) or [LSC][2] (delta: g, beta)
+    float* v_s = a_s + LSC * (DELTA ? 2 : d);  // [LSC][VT]
+    for (int t0 = b; t0 < e; t0 += LSC) {
+      const int nt = (e - t0 < LSC) ? e - t0 : LSC;
+      __syncthreads();
+      for (int idx = tid; idx < nt * d; idx += nthreads) {
+        const int tt = idx / d, n = idx - tt * d;
+        const int64_t t = t0 + tt;
+        const int at = FULL ? tt * d + (n % NSL) * NPT + n / NSL : idx;
+        q_s[at] = q[t * q_stride + hk * d + n] * q_scale;
+        k_s[at] = k[t * k_stride + hk * d + n];
+        if (!DELTA) a_s[at] = decay[t * decay_stride + h * d + n];
+      }
+      if (DELTA) {
+        for (int tt = tid; tt < nt; tt += nthreads) {
+          a_s[2 * tt] = decay[static_cast<int64_t>(t0 + tt) * decay_stride + h];
+          a_s[2 * tt + 1] = beta[static_cast<int64_t>(t0 + tt) * beta_stride + h];
+        }
+      }
+      for (int idx = tid; idx < nt * VT; idx += nthreads) {
+        const int tt = idx / VT, cc = c0 + idx - tt * VT;
+        v_s[idx] = cc < dv ? v[static_cast<int64_t>(t0 + tt) * v_stride + h * dv + cc] : 0.f;
+      }
+      __syncthreads();
+      work_stage(q_s, k_s, a_s, v_s, t0, nt);
+    }
   }
   if (!c_ok) return;
 #pragma unroll
   for (int i = 0; i < NPT; ++i) {
     const int n = ns + NSL * i;
-    if (n < d) st[static_cast<int64_t>(n) * dv + c] = s[i];
+    if (n < d) st[st_at(n)] = s[i];
   }
 }
 
@@ -265,17 +339,22 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   if (grid.y > 65535u || grid.z > 65535u) return kvc_fail("kvc_linear_state_scan: grid too large");
   const size_t lds = sizeof(float) * (2 * LSC * d + LSC * (delta_rule ? 2 : d) + LSC * VT);
   const int per_thread = (d + NSL - 1) / NSL;
-#define KVC_LSCAN_F(NPT, DELTA, NSL_, FULL_)                                                                  \
-  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_>), grid, dim3(256), lds, S(stream), out, \
-                     q, q_stride, k, k_stride, v, v_stride, decay, decay_stride, beta, beta_stride, state,    \
-                     positions, token_req, q_start, slots, nh, nqk, d, dv, q_scale)
-#define KVC_LSCAN(NPT, DELTA, NSL_)        \
-  do {                                     \
-    if (d == NPT * NSL_) {                 \
-      KVC_LSCAN_F(NPT, DELTA, NSL_, 1);    \
-    } else {                               \
-      KVC_LSCAN_F(NPT, DELTA, NSL_, 0);    \
-    }                                      \
+#define KVC_LSCAN_F(NPT, DELTA, NSL_, FULL_, PF_)                                                             \
+  hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_, PF_>), grid, dim3(256),               \
+                     lds*(PF_ ? 2 : 1), S(stream), out, q, q_stride, k, k_stride, v, v_stride, decay,         \
+                     decay_stride, beta, beta_stride, state, positions, token_req, q_start, slots, nh, nqk, d, \
+                     dv, q_scale)
+  // two sets of LDS buffers (the next stage fetched while one is worked on) where a stage's values
+  // deal out evenly to the threads and both sets fit the 64 KB a block may take
+#define KVC_LSCAN(NPT, DELTA, NSL_)                                                  \
+  do {                                                                               \
+    if (d == NPT * NSL_ && (NPT * NSL_) % 16 == 0 && 2 * lds <= 64 * 1024) {         \
+      KVC_LSCAN_F(NPT, DELTA, NSL_, 1, ((NPT * NSL_) % 16 == 0 ? 1 : 0));            \
+    } else if (d == NPT * NSL_) {                                                    \
+      KVC_LSCAN_F(NPT, DELTA, NSL_, 1, 0);                                           \
+    } else {                                                                         \
+      KVC_LSCAN_F(NPT, DELTA, NSL_, 0, 0);                                           \
+    }                                                                                \
   } while (0)
 #define KVC_LSCAN_N(NPT)                 \
   do {                                   \

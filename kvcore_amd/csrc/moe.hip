@@ -175,24 +175,26 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
 #pragma unroll
         for (int i = 0; i < 4; ++i) xv[j][i] = (k + i < H) ? to_float(xr[i]) : 0.f;
       }
+      // every expert's piece is asked for before any is used, with no branch between the loads
+      // (an expert beyond the last reads the last one's row again; its sums are dropped)
+      float wv[EB][4];
 #pragma unroll
       for (int e = 0; e < EB; ++e) {
-        if (e < ne) {
-          const float* wp = wr + static_cast<int64_t>(e0 + e) * H + k;
-          float wv[4];
-          if (vectors) {
-            const float4 v4 = *reinterpret_cast<const float4*>(wp);
-            wv[0] = v4.x; wv[1] = v4.y; wv[2] = v4.z; wv[3] = v4.w;
-          } else {
+        const float* wp = wr + static_cast<int64_t>(e < ne ? e0 + e : E - 1) * H + k;
+        if (vectors) {
+          const float4 v4 = *reinterpret_cast<const float4*>(wp);
+          wv[e][0] = v4.x; wv[e][1] = v4.y; wv[e][2] = v4.z; wv[e][3] = v4.w;
+        } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) wv[i] = (k + i < H) ? wp[i] : 0.f;
-          }
-#pragma unroll
-          for (int j = 0; j < TOK; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[j][e] = fmaf(xv[j][i], wv[i], acc[j][e]);
+          for (int i = 0; i < 4; ++i) wv[e][i] = (k + i < H) ? wp[i] : 0.f;
         }
       }
+#pragma unroll
+      for (int e = 0; e < EB; ++e)
+#pragma unroll
+        for (int j = 0; j < TOK; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[j][e] = fmaf(xv[j][i], wv[e][i], acc[j][e]);
     }
 #pragma unroll
     for (int j = 0; j < TOK; ++j) {

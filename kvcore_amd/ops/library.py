@@ -1242,6 +1242,12 @@ def _f32_rows(t: torch.Tensor, name: str, cols: int) -> tuple[int, int]:
     return ptr, stride
 
 
+def linear_state_rows(dim: int) -> int:
+    """Rows of a head's state as ``linear_state_scan`` keeps it: ``dim`` rounded up to a multiple of 4
+    (the kernel lays the rows out in fours)."""
+    return -(-dim // 4) * 4
+
+
 def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       decay: torch.Tensor, beta: torch.Tensor | None, state: torch.Tensor, *,
                       positions: torch.Tensor, token_req: torch.Tensor, q_start: torch.Tensor,
@@ -1250,13 +1256,15 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
     """The recurrence of a matrix state per head (see the C header): ``q, k [T, qk_heads * dim]``,
     ``v [T, heads * vdim]``, all float32 rows (column views are fine); ``decay [T, heads * dim]``
     (a factor per key channel) or, with ``delta_rule``, ``decay`` and ``beta [T, heads]``;
-    ``state [slots, heads, dim, vdim]`` float32; ``out [T, heads * vdim]`` float32.  ``q_scale``
+    ``state [slots, heads, linear_state_rows(dim), vdim]`` float32, in an order of the kernel's own;
+    ``out [T, heads * vdim]`` float32.  ``q_scale``
     multiplies every q on its way in."""
     T = out.shape[0]
     if out.shape != (T, heads * vdim) or not out.is_contiguous() or out.dtype != torch.float32:
         raise KernelError("linear_state_scan: out must be contiguous float32 [T, heads * vdim]")
-    if tuple(state.shape[1:]) != (heads, dim, vdim) or state.dtype != torch.float32 or not state.is_contiguous():
-        raise KernelError("linear_state_scan: state must be float32 [slots, heads, dim, vdim]")
+    if tuple(state.shape[1:]) != (heads, linear_state_rows(dim), vdim) or state.dtype != torch.float32 \
+            or not state.is_contiguous():
+        raise KernelError("linear_state_scan: state must be float32 [slots, heads, linear_state_rows(dim), vdim]")
     if min(q.shape[0], k.shape[0], v.shape[0], decay.shape[0]) < T or positions.numel() < T \
             or token_req.numel() < T or q_start.numel() < num_reqs + 1:
         raise KernelError("linear_state_scan: rows or index arrays too short")

@@ -100,7 +100,7 @@ class GatedLinearAttention(_MatrixStateMixer):
         return ("in_proj.weight", "o.weight")
 
     def state_needs(self) -> tuple[StateNeed, ...]:
-        return (StateNeed((self.heads, self.dim, self.vdim)),)
+        return (StateNeed((self.heads, ops.linear_state_rows(self.dim), self.vdim)),)
 
     def forward(self, x, ctx, call, sink=None):
         p, qk, inner = self.params, self.qk, self.inner
@@ -165,7 +165,8 @@ class GatedDeltaRule(_MatrixStateMixer):
 
     def state_needs(self) -> tuple[StateNeed, ...]:
         # the convolution's last inputs (at least one row, so that the array exists), the matrices
-        return (StateNeed((max(self.taps - 1, 1), self.conv_dim)), StateNeed((self.heads, self.dim, self.vdim)))
+        return (StateNeed((max(self.taps - 1, 1), self.conv_dim)),
+                StateNeed((self.heads, ops.linear_state_rows(self.dim), self.vdim)))
 
     def forward(self, x, ctx, call, sink=None):
         p, qk, inner, nh = self.params, self.qk, self.inner, self.heads

@@ -27,6 +27,13 @@ def rel(got, want):
 
 
 # ------------------------------------------------------------------ the matrix state
+def new_state(slots, heads, dim, vdim, fill=float("nan")):
+    """Slots as the engine keeps them (NaN where a request must not read: another's leftovers)."""
+    from kvcore_amd.ops import library as ops
+
+    return torch.full((slots, heads, ops.linear_state_rows(dim), vdim), fill, device=DEV)
+
+
 def run_scan(q, k, v, decay, beta, state, reqs, *, heads, qk_heads, dim, vdim, delta, q_scale=1.0):
     from kvcore_amd.ops import library as ops
 
@@ -51,11 +58,11 @@ def test_key_decay_recurrence_whole_in_steps_and_beside_others(heads, qk_heads, 
     qg, kg, vg, ag = (gpu(t.reshape(T, -1)) for t in (q, k, v, a))
     kw = dict(heads=heads, qk_heads=qk_heads, dim=dim, vdim=vdim, delta=False, q_scale=0.3)
     # the slots hold another request's leftovers (NaN where nothing may be read)
-    state = torch.full((3, heads, dim, vdim), float("nan"), device=DEV)
+    state = new_state(3, heads, dim, vdim)
     out = run_scan(qg, kg, vg, ag, None, state, [(1, 0, T)], **kw)
     assert rel(out, want) < 2e-6
     # in steps of every size down to one token, cut inside the stages of 16
-    state = torch.full((3, heads, dim, vdim), float("nan"), device=DEV)
+    state = new_state(3, heads, dim, vdim)
     at, got = 0, []
     for n in (2, 1, 17, 3, 1, 16, 31, 2, 10):
         got.append(run_scan(qg[at:at + n], kg[at:at + n], vg[at:at + n], ag[at:at + n], None, state, [(2, at, n)], **kw))
@@ -63,7 +70,7 @@ def test_key_decay_recurrence_whole_in_steps_and_beside_others(heads, qk_heads, 
     assert at == T
     assert rel(torch.cat(got), want) < 2e-6
     # beside a padded row and another request that is further on: rows [other | pad | this]
-    other = torch.zeros((3, heads, dim, vdim), device=DEV)
+    other = new_state(3, heads, dim, vdim, 0.0)
     mixed_q = torch.cat([qg[40:41], qg[:1], qg[:20]])
     mixed_k = torch.cat([kg[40:41], kg[:1], kg[:20]])
     mixed_v = torch.cat([vg[40:41], vg[:1], vg[:20]])
@@ -90,10 +97,10 @@ def test_delta_rule_whole_in_steps_and_beside_others(heads, qk_heads, dim, vdim)
     qg, kg, vg = (gpu(t.reshape(T, -1)) for t in (q, k, v))
     bg, gg = gpu(beta), gpu(g)
     kw = dict(heads=heads, qk_heads=qk_heads, dim=dim, vdim=vdim, delta=True)
-    state = torch.full((2, heads, dim, vdim), float("nan"), device=DEV)
+    state = new_state(2, heads, dim, vdim)
     out = run_scan(qg, kg, vg, gg, bg, state, [(1, 0, T)], **kw)
     assert rel(out, want) < 5e-6
-    state = torch.full((2, heads, dim, vdim), float("nan"), device=DEV)
+    state = new_state(2, heads, dim, vdim)
     at, got = 0, []
     for n in (1, 2, 16, 1, 19, 2, 29):
         got.append(run_scan(qg[at:at + n], kg[at:at + n], vg[at:at + n], gg[at:at + n], bg[at:at + n], state,
@@ -104,7 +111,7 @@ def test_delta_rule_whole_in_steps_and_beside_others(heads, qk_heads, dim, vdim)
     # a column view of a wider row, as the mixers hand their projections over
     wide = torch.cat([qg, kg, vg], dim=1).contiguous()
     nq = qk_heads * dim
-    state = torch.zeros((2, heads, dim, vdim), device=DEV)
+    state = new_state(2, heads, dim, vdim, 0.0)
     out = run_scan(wide[:, :nq], wide[:, nq:2 * nq], wide[:, 2 * nq:], gg, bg, state, [(0, 0, T)], **kw)
     assert rel(out, want) < 5e-6
 
@@ -127,10 +134,10 @@ def test_a_token_written_six_hundred_tokens_ago_is_still_read():
     assert torch.allclose(want[600], v[0, 0] * 0.999 ** 600, atol=1e-9)
     qg, kg, vg, ag = (gpu(t.reshape(T, -1)) for t in (q, k, v, a))
     kw = dict(heads=1, qk_heads=1, dim=d, vdim=dv, delta=False)
-    state = torch.full((1, 1, d, dv), float("nan"), device=DEV)
+    state = new_state(1, 1, d, dv)
     out = run_scan(qg, kg, vg, ag, None, state, [(0, 0, T)], **kw)
     assert rel(out[600], want[600]) < 1e-4
-    state = torch.full((1, 1, d, dv), float("nan"), device=DEV)
+    state = new_state(1, 1, d, dv)
     run_scan(qg[:300], kg[:300], vg[:300], ag[:300], None, state, [(0, 0, 300)], **kw)
     for t in range(300, T):
         out = run_scan(qg[t:t + 1], kg[t:t + 1], vg[t:t + 1], ag[t:t + 1], None, state, [(0, t, 1)], **kw)
