@@ -87,10 +87,22 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   auto st_at = [&](int n) -> int64_t { return (static_cast<int64_t>(n >> 2) * dv + c) * 4 + (n & 3); };
   const bool fresh = positions[b] == 0;
   float s[NPT];
+  if (!fresh) {  // the same for the whole block
+    // every row is asked for with no branch between the loads (a row or column that is not there
+    // reads one that is, and is then set to zero), so that all of them are in flight together
+    const int c_safe = c_ok ? c : dv - 1;
 #pragma unroll
-  for (int i = 0; i < NPT; ++i) {
-    const int n = ns + NSL * i;
-    s[i] = (!fresh && c_ok && n < d) ? st[st_at(n)] : 0.f;
+    for (int i = 0; i < NPT; ++i) {
+      const int n = ns + NSL * i;
+      const int n_safe = (FULL || n < d) ? n : 0;
+      s[i] = st[(static_cast<int64_t>(n_safe >> 2) * dv + c_safe) * 4 + (n_safe & 3)];
+    }
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      if (!c_ok || !(FULL || ns + NSL * i < d)) s[i] = 0.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) s[i] = 0.f;
   }
   // one stage's tokens, from the LDS buffers given
   auto work_stage = [&](const float* q_s, const float* k_s, const float* a_s, const float* v_s, int t0, int nt) {

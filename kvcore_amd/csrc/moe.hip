@@ -280,8 +280,8 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int li = lane & 15, lk = lane >> 4;
   // B operand: token row li of the tile; A operand: the expert's row n0 + li
   const bool row_ok = li < nr;
-  const int pair = row_ok ? sorted[r0 + li] : 0;
-  const int64_t in_row = in_div > 0 ? pair / in_div : r0 + li;
+  const int pair = sorted[r0 + (row_ok ? li : 0)];
+  const int64_t in_row = in_div > 0 ? pair / in_div : r0 + (row_ok ? li : 0);
   const bf16_t* xr = x + in_row * x_stride + 16 * lk;
   const int wrow = n0 + li < N ? n0 + li : N - 1;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     for (int h = 0; h < 2; ++h) {
       an[h] = *reinterpret_cast<const bf16x8_t*>(wr + k + 8 * h);
       if (GATED) a2n[h] = *reinterpret_cast<const bf16x8_t*>(wr2 + k + 8 * h);
-      bn[h] = row_ok ? *reinterpret_cast<const bf16x8_t*>(xr + k + 8 * h) : zero8();
+      bn[h] = *reinterpret_cast<const bf16x8_t*>(xr + k + 8 * h);  // a row that is not there reads the tile's first
     }
   };
   if (k_main > 0) fetch(0);
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     for (int h = 0; h < 2; ++h) {
       a[h] = an[h];
       if (GATED) a2[h] = a2n[h];
-      b[h] = bn[h];
+      b[h] = row_ok ? bn[h] : zero8();
     }
     if (k + 64 < k_main) fetch(k + 64);
 #pragma unroll
@@ -366,8 +366,8 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
   // staging: thread t brings 8 values of row t / 4 of the tile
   const int srow = threadIdx.x >> 2, spart = threadIdx.x & 3;
   const bool srow_ok = srow < nr;
-  int64_t in_row = 0;
-  if (srow_ok) in_row = in_div > 0 ? sorted[r0 + srow] / in_div : r0 + srow;
+  const int srow_safe = srow_ok ? srow : 0;  // a row that is not there reads the tile's first, and is set to zero
+  const int64_t in_row = in_div > 0 ? sorted[r0 + srow_safe] / in_div : r0 + srow_safe;
   const bf16_t* xp = x + in_row * x_stride + 8 * spart;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
   const bf16_t* wp[NF];
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
   uint4 x_next = uint4{0u, 0u, 0u, 0u};
   bf16x8_t w_next[NF], w2_next[GATED ? NF : 1];
   auto fetch = [&](int k) {
-    if (srow_ok) x_next = *reinterpret_cast<const uint4*>(xp + k);
+    x_next = *reinterpret_cast<const uint4*>(xp + k);
     if (wave_live) {
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
   fetch(0);
   for (int k = 0; k < K; k += 32) {
     __syncthreads();  // the chunk before has been read by every wave
-    *reinterpret_cast<uint4*>(x_s + srow * KROW + 8 * spart) = x_next;
+    *reinterpret_cast<uint4*>(x_s + srow * KROW + 8 * spart) = srow_ok ? x_next : uint4{0u, 0u, 0u, 0u};
     bf16x8_t wa[NF], wa2[GATED ? NF : 1];
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
