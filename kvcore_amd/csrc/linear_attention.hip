@@ -15,6 +15,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "device_utils.h"
 #include "kvcore_hip.h"
 
@@ -351,6 +353,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   if (grid.y > 65535u || grid.z > 65535u) return kvc_fail("kvc_linear_state_scan: grid too large");
   const size_t lds = sizeof(float) * (2 * LSC * d + LSC * (delta_rule ? 2 : d) + LSC * VT);
   const int per_thread = (d + NSL - 1) / NSL;
+  static const bool no_pf = getenv("KVC_LSCAN_NOPF") != nullptr;  // for tuning
 #define KVC_LSCAN_F(NPT, DELTA, NSL_, FULL_, PF_)                                                             \
   hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_, PF_>), grid, dim3(256),               \
                      lds*(PF_ ? 2 : 1), S(stream), out, q, q_stride, k, k_stride, v, v_stride, decay,         \
@@ -360,7 +363,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   // deal out evenly to the threads and both sets fit the 64 KB a block may take
 #define KVC_LSCAN(NPT, DELTA, NSL_)                                                  \
   do {                                                                               \
-    if (d == NPT * NSL_ && (NPT * NSL_) % 16 == 0 && 2 * lds <= 64 * 1024) {         \
+    if (d == NPT * NSL_ && (NPT * NSL_) % 16 == 0 && 2 * lds <= 64 * 1024 && !no_pf) {  \
       KVC_LSCAN_F(NPT, DELTA, NSL_, 1, ((NPT * NSL_) % 16 == 0 ? 1 : 0));            \
     } else if (d == NPT * NSL_) {                                                    \
       KVC_LSCAN_F(NPT, DELTA, NSL_, 1, 0);                                           \

@@ -144,10 +144,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ ch
 }
 
 // The router whole: logits = x W^T in float32 (x of either dtype, its values as they are), then the
-// choice as in moe_route_kernel.  A wave takes TOK tokens: lane l sums the products of the values
-// 4 l .. 4 l + 3 of every 256 along K for each of up to 32 experts at a time (a fetched piece of the
-// router's row meets all TOK tokens), the 64 partial sums of a logit are added in lane order through
-// LDS: one fixed order, whatever the batch.
+// choice as in moe_route_kernel.  A block takes TOK tokens.  Its four waves share K: lane l of wave
+// w sums the products of the values 4 l .. 4 l + 3 of the pieces of 256 that are the wave's (every
+// fourth piece) for each of up to 32 experts at a time (a fetched piece of the router's row meets all
+// TOK tokens); the 256 partial sums of a logit are added in wave and lane order through LDS: one
+// fixed order, whatever the batch.  The first wave then chooses.
 template <typename T, int TOK>
 __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
                                                          const T* __restrict__ x, int64_t x_stride,
@@ -156,10 +157,9 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
   constexpr int EB = 32, PR = EB + 1;
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  float* part = lds + wave * (kWave * PR);                               // [64][EB + 1]
-  float* z = lds + 4 * kWave * PR + wave * TOK * (E + groups);           // [TOK][E + groups]
-  const int t0 = (blockIdx.x * 4 + wave) * TOK;
-  if (t0 >= T_) return;  // the whole wave
+  float* part = lds;                       // [256][EB + 1]
+  float* z = lds + 256 * PR;               // [TOK][E + groups]
+  const int t0 = blockIdx.x * TOK;
   for (int e0 = 0; e0 < E; e0 += EB) {
     const int ne = (E - e0 < EB) ? E - e0 : EB;
     float acc[TOK][EB];
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
     for (int j = 0; j < TOK; ++j)
 #pragma unroll
       for (int e = 0; e < EB; ++e) acc[j][e] = 0.f;
-    for (int k = 4 * lane; k < H; k += 4 * kWave) {
+    for (int k = 4 * lane + 4 * kWave * wave; k < H; k += 16 * kWave) {
       float xv[TOK][4];
 #pragma unroll
       for (int j = 0; j < TOK; ++j) {
@@ -198,17 +198,19 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
     }
 #pragma unroll
     for (int j = 0; j < TOK; ++j) {
+      __syncthreads();  // the partial sums of the token before have been added up
 #pragma unroll
-      for (int e = 0; e < EB; ++e) part[lane * PR + e] = acc[j][e];
-      __builtin_amdgcn_wave_barrier();
-      if (lane < ne) {
+      for (int e = 0; e < EB; ++e) part[threadIdx.x * PR + e] = acc[j][e];
+      __syncthreads();
+      if (threadIdx.x < ne) {
         float sum = 0.f;
-        for (int l = 0; l < kWave; ++l) sum += part[l * PR + lane];
-        z[j * (E + groups) + e0 + lane] = sum;
+        for (int l = 0; l < 256; ++l) sum += part[l * PR + threadIdx.x];
+        z[j * (E + groups) + e0 + threadIdx.x] = sum;
       }
-      __builtin_amdgcn_wave_barrier();
     }
   }
+  __syncthreads();
+  if (wave != 0) return;
   for (int j = 0; j < TOK; ++j) {
     const int t = t0 + j;
     if (t >= T_) break;  // the whole wave
@@ -518,12 +520,12 @@ extern "C" int kvc_moe_router(int32_t* choice, float* weight, const void* x, int
       keep > groups || x_stride < H)
     return kvc_fail("kvc_moe_router: bad sizes (at most 64 choices; the experts in equal groups)");
   if (T == 0) return 0;
-  // four tokens a wave where the waves then still fill the chip, else one
-  const bool big = T >= 4 * 4 * kvc_device_compute_units();
+  // four tokens a block where the blocks then still fill the chip several times over, else one
+  const bool big = T >= 4 * 8 * kvc_device_compute_units();
   const int TOK = big ? 4 : 1;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(4) * 64 * 33 + static_cast<size_t>(4) * TOK * (E + groups));
+  const size_t lds = sizeof(float) * (static_cast<size_t>(256) * 33 + static_cast<size_t>(TOK) * (E + groups));
   if (lds > 160 * 1024) return kvc_fail("kvc_moe_router: too many experts for a block's LDS");
-  const dim3 grid((T + 4 * TOK - 1) / (4 * TOK));
+  const dim3 grid((T + TOK - 1) / TOK);
   // 16-byte loads of the router's rows where the rows allow
   const int vectors = H % 4 == 0 && (reinterpret_cast<uintptr_t>(router) & 15) == 0;
 #define KVC_ROUTER(Tp, TOK_)                                                                                    \
