@@ -240,7 +240,8 @@ int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* 
 // kvc_moe_gemm multiplies every tile's rows by its expert's matrix: w is [E, N, K], or with
 // `gated` [E, 2N, K] (gate rows, then up rows) and the activation applied; a sorted row i reads
 // x row sorted[i] / in_div (in_div 0: row i itself) and writes out row i (out_sorted) or
-// sorted[i].  dtype is that of x and w.
+// sorted[i].  dtype is that of x and w.  packed: w is the copy kvc_pack_weight makes of the whole
+// stacked matrix (bfloat16, tiles of 16 rows only, N a multiple of 16, K of 64).
 int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
                   int groups, int keep, kvc_stream stream);
 // Tiles hold up to tile_rows rows, 16 or 64 (kvc_moe_tile_rows says which a step's size asks
@@ -256,7 +257,7 @@ int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int
 int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                  const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
                  const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div, int out_sorted,
-                 int gated, float limit, float alpha, kvc_stream stream);
+                 int gated, float limit, float alpha, int packed, kvc_stream stream);
 // out[t] = sum_c weight[t, c] * y[t * top + c] + add0[t] + add1[t] (either may be null; add0 of
 // dtype add0_dtype, add1 float32), float32.
 int kvc_moe_combine(float* out, const float* y, const float* weight, int top, const void* add0,

@@ -266,9 +266,9 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
 // 64 values along K: lane (li, lk) fetches the 16 values from 16 lk of its weight row and of its
 // token row (32 contiguous bytes, so that the four lanes of a row read one 128-byte line) and the two
 // matrix instructions of the round take its first and its second eight (both operands are dealt the
-// same way, so each product still sums over all of K); the next round's values are asked for
+// same way, so each product still sums over all of K); the next two rounds' values are asked for
 // before this round's products.
-template <int GATED, typename TO>
+template <int GATED, typename TO, int PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
     const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
@@ -284,36 +284,61 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const bool row_ok = li < nr;
   const int pair = sorted[r0 + (row_ok ? li : 0)];
   const int64_t in_row = in_div > 0 ? pair / in_div : r0 + (row_ok ? li : 0);
-  const bf16_t* xr = x + in_row * x_stride + 16 * lk;
+  // PACKED: w is the copy that `kvc_pack_weight` makes, tiles of 16 rows x 32 values of K in one
+  // piece of 1 KB each, so a wave's load of an operand is one contiguous kilobyte instead of 128 bytes
+  // from each of 16 rows that lie 2 K bytes apart (which meet in the same memory channels); the lanes
+  // then take K in the plain order, 8 values from 8 lk of each 32.
+  const bf16_t* xr = x + in_row * x_stride + (PACKED ? 8 : 16) * lk;
   const int wrow = n0 + li < N ? n0 + li : N - 1;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
-  const bf16_t* wr = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 16 * lk;
-  const bf16_t* wr2 = wr + static_cast<int64_t>(N) * K;  // the up rows follow the gate rows
+  const bf16_t* wr = PACKED ? w + ((static_cast<int64_t>(e) * rows_per_expert + n0) >> 4) * (K / 32) * 512 + li * 32 + lk * 8
+                            : w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 16 * lk;
+  const bf16_t* wr2 = wr + static_cast<int64_t>(N) * K;  // the up rows follow the gate rows (in either order of storage)
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
   const int k_main = K & ~63;
-  bf16x8_t an[2], a2n[2], bn[2];
-  auto fetch = [&](int k) {
+  // two rounds are on their way while one is multiplied
+  bf16x8_t an[2][2], a2n[2][2], bn[2][2];
+  auto fetch = [&](int k, int slot) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      an[h] = *reinterpret_cast<const bf16x8_t*>(wr + k + 8 * h);
-      if (GATED) a2n[h] = *reinterpret_cast<const bf16x8_t*>(wr2 + k + 8 * h);
-      bn[h] = *reinterpret_cast<const bf16x8_t*>(xr + k + 8 * h);  // a row that is not there reads the tile's first
+      const int64_t wo = PACKED ? static_cast<int64_t>(k / 32 + h) * 512 : k + 8 * h;
+      an[slot][h] = *reinterpret_cast<const bf16x8_t*>(wr + wo);
+      if (GATED) a2n[slot][h] = *reinterpret_cast<const bf16x8_t*>(wr2 + wo);
+      // a row that is not there reads the tile's first
+      bn[slot][h] = *reinterpret_cast<const bf16x8_t*>(xr + k + (PACKED ? 32 : 8) * h);
     }
   };
-  if (k_main > 0) fetch(0);
-  for (int k = 0; k < k_main; k += 64) {
-    bf16x8_t a[2], a2[2], b[2];
+  if (k_main > 0) fetch(0, 0);
+  if (k_main > 64) fetch(64, 1);
+  for (int k = 0; k < k_main; k += 128) {
+    // slot 0 holds round k, slot 1 round k + 64; each is asked for again as soon as it has been used
+    bf16x8_t a0[2], a20[2], b0[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      a[h] = an[h];
-      if (GATED) a2[h] = a2n[h];
-      b[h] = row_ok ? bn[h] : zero8();
+      a0[h] = an[0][h];
+      if (GATED) a20[h] = a2n[0][h];
+      b0[h] = row_ok ? bn[0][h] : zero8();
     }
-    if (k + 64 < k_main) fetch(k + 64);
+    if (k + 128 < k_main) fetch(k + 128, 0);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h], b[h], acc, 0, 0, 0);
-      if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[h], b[h], acc2, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[h], b0[h], acc, 0, 0, 0);
+      if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a20[h], b0[h], acc2, 0, 0, 0);
+    }
+    if (k + 64 < k_main) {
+      bf16x8_t a1[2], a21[2], b1[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        a1[h] = an[1][h];
+        if (GATED) a21[h] = a2n[1][h];
+        b1[h] = row_ok ? bn[1][h] : zero8();
+      }
+      if (k + 192 < k_main) fetch(k + 192, 1);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[h], b1[h], acc, 0, 0, 0);
+        if (GATED) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a21[h], b1[h], acc2, 0, 0, 0);
+      }
     }
   }
   if (k_main < K) {  // a ragged end along K (a multiple of 8): element by element, zeros beyond
@@ -570,7 +595,7 @@ extern "C" int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles
 extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                             const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
                             const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div,
-                            int out_sorted, int gated, float limit, float alpha, kvc_stream stream) {
+                            int out_sorted, int gated, float limit, float alpha, int packed, kvc_stream stream) {
   if (max_tiles < 0 || N <= 0 || K <= 0 || x_stride < K || out_stride < N)
     return kvc_fail("kvc_moe_gemm: bad sizes");
   if (tile_rows != kTileRows && tile_rows != kBigTileRows) return kvc_fail("kvc_moe_gemm: tiles of 16 or 64 rows");
@@ -587,17 +612,25 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
     const bool vectors = K % 8 == 0 && x_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(w) & 15) == 0;
     if (tile_rows == kBigTileRows) {
+      if (packed) return kvc_fail("kvc_moe_gemm: tiles of 64 rows read the matrix row by row");
       if (!vectors || K % 32) return kvc_fail("kvc_moe_gemm: tiles of 64 rows need K to be a multiple of 32");
       grid.y = gated ? (N + 127) / 128 : (N + 255) / 256;
       if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, bf16_t>), bf16_t, bf16_t);
       else if (gated) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, float>), bf16_t, float);
       else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, bf16_t>), bf16_t, bf16_t);
       else KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, float>), bf16_t, float);
+    } else if (packed) {
+      if (!vectors || N % 16 || K % 64)
+        return kvc_fail("kvc_moe_gemm: a packed matrix has experts of a multiple of 16 rows of a multiple of 64");
+      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, bf16_t, 1>), bf16_t, bf16_t);
+      else if (gated) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, float, 1>), bf16_t, float);
+      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, bf16_t, 1>), bf16_t, bf16_t);
+      else KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, float, 1>), bf16_t, float);
     } else if (vectors) {
-      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, bf16_t>), bf16_t, bf16_t);
-      else if (gated) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, float>), bf16_t, float);
-      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, bf16_t>), bf16_t, bf16_t);
-      else KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, float>), bf16_t, float);
+      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, bf16_t, 0>), bf16_t, bf16_t);
+      else if (gated) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<1, float, 0>), bf16_t, float);
+      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, bf16_t, 0>), bf16_t, bf16_t);
+      else KVC_MOE_LAUNCH((moe_gemm_bf16_kernel<0, float, 0>), bf16_t, float);
     } else {
       if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, bf16_t, bf16_t>), bf16_t, bf16_t);
       else if (gated) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, bf16_t, float>), bf16_t, float);
@@ -606,7 +639,7 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
     }
   } else if (dtype == 0) {
     if (out_dtype != 0) return kvc_fail("kvc_moe_gemm: float32 operands give float32 rows");
-    if (tile_rows != kTileRows) return kvc_fail("kvc_moe_gemm: float32 operands take tiles of 16 rows");
+    if (tile_rows != kTileRows || packed) return kvc_fail("kvc_moe_gemm: float32 operands take tiles of 16 rows of a row-major matrix");
     if (gated) KVC_MOE_LAUNCH((moe_gemm_plain_kernel<1, float, float>), float, float);
     else KVC_MOE_LAUNCH((moe_gemm_plain_kernel<0, float, float>), float, float);
   } else {

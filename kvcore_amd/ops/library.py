@@ -58,7 +58,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_moe_max_tiles": [I, I, I],
         "kvc_moe_tile_rows": [I, I],
         "kvc_moe_align": [P, P, P, P, I, I, I, I, P],
-        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, P],
+        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, P],
         "kvc_clamped_glu": [P, P, I, I, F, F, I, P],
         "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
@@ -1392,11 +1392,13 @@ def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: 
     if w.shape != (rows, K) or out.shape[0] < pairs or x.dtype != w.dtype or out.stride(1) != 1 or x.stride(1) != 1:
         raise KernelError("moe_gemm: shapes do not match")
     max_tiles = min(tiles.shape[0], moe_max_tiles(pairs, experts, tile_rows))
+    # single tokens stream the packed twin of the experts' matrix where the model keeps one
+    w_ptr, packed = (_streamed(w, N) if tile_rows == 16 and N % 16 == 0 and K % 64 == 0 else (_dev(w, "w"), 0))
     _check(load().kvc_moe_gemm(out.data_ptr(), out.stride(0), _code(out, "out"), x.data_ptr(), x.stride(0),
-                               _dev(w, "w"), _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
+                               w_ptr, _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
                                _dev(tiles, "tiles", torch.int32), _dev(num_tiles, "num_tiles", torch.int32),
                                max_tiles, tile_rows, N, K, int(in_div), int(bool(out_sorted)), int(bool(gated)),
-                               float(limit), float(alpha), _stream()), "kvc_moe_gemm")
+                               float(limit), float(alpha), packed, _stream()), "kvc_moe_gemm")
 
 
 def moe_combine(out: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, add0: torch.Tensor | None = None,

@@ -68,7 +68,9 @@ class RoutedExperts(FeedForward):
         return specs
 
     def product_weights(self) -> tuple[str, ...]:
-        return ("shared.gate_up", "shared.down") if self.shared_size else ()
+        # the experts' stacked matrices too: steps of single tokens stream their packed twins
+        shared = ("shared.gate_up", "shared.down") if self.shared_size else ()
+        return ("experts.gate_up", "experts.down", *shared)
 
     def forward(self, x, ctx, call, sink=None):
         p, H, E, I, top = self.params, self.hidden_size, self.experts, self.expert_size, self.top
