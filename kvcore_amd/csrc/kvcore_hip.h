@@ -241,7 +241,7 @@ int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* 
 // `gated` [E, 2N, K] (gate rows, then up rows) and the activation applied; a sorted row i reads
 // x row sorted[i] / in_div (in_div 0: row i itself) and writes out row i (out_sorted) or
 // sorted[i].  dtype is that of x and w.  packed: w is the copy kvc_pack_weight makes of the whole
-// stacked matrix (bfloat16, tiles of 16 rows only, N a multiple of 16, K of 64).
+// stacked matrix (bfloat16, N a multiple of 16, K of 64).
 int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
                   int groups, int keep, kvc_stream stream);
 // Tiles hold up to tile_rows rows, 16 or 64 (kvc_moe_tile_rows says which a step's size asks

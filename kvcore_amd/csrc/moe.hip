@@ -374,7 +374,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
 // the B operand (four row blocks of 16); every wave fetches the weight rows of its own columns
 // straight into registers as the A operand (NF blocks of 16 columns, for gate and for up), one
 // chunk ahead of the products.  Every fetched weight meets 64 rows, every row 128 or 256 columns.
-template <int GATED, typename TO>
+template <int GATED, typename TO, int PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
     const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
@@ -401,7 +401,10 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
 #pragma unroll
   for (int f = 0; f < NF; ++f) {
     const int wrow = n0 + 16 * f + li < N ? n0 + 16 * f + li : N - 1;
-    wp[f] = w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 8 * lk;
+    // PACKED (N a multiple of 16): the copy in pieces of 16 rows x 32 values, one contiguous kilobyte a load
+    const int ntile = n0 + 16 * f < N ? n0 + 16 * f : N - 16;
+    wp[f] = PACKED ? w + ((static_cast<int64_t>(e) * rows_per_expert + ntile) >> 4) * (K / 32) * 512 + li * 32 + lk * 8
+                   : w + (static_cast<int64_t>(e) * rows_per_expert + wrow) * K + 8 * lk;
   }
   const int64_t up_off = static_cast<int64_t>(N) * K;
   f32x4_t acc[NF][NR], acc2[GATED ? NF : 1][NR];
@@ -419,8 +422,9 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     if (wave_live) {
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
-        w_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + k);
-        if (GATED) w2_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + up_off + k);
+        const int64_t wo = PACKED ? static_cast<int64_t>(k / 32) * 512 : k;
+        w_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + wo);
+        if (GATED) w2_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + up_off + wo);
       }
     }
   };
@@ -612,13 +616,21 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
     const bool vectors = K % 8 == 0 && x_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(w) & 15) == 0;
     if (tile_rows == kBigTileRows) {
-      if (packed) return kvc_fail("kvc_moe_gemm: tiles of 64 rows read the matrix row by row");
       if (!vectors || K % 32) return kvc_fail("kvc_moe_gemm: tiles of 64 rows need K to be a multiple of 32");
+      if (packed && (N % 16 || K % 64))
+        return kvc_fail("kvc_moe_gemm: a packed matrix has experts of a multiple of 16 rows of a multiple of 64");
       grid.y = gated ? (N + 127) / 128 : (N + 255) / 256;
-      if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, bf16_t>), bf16_t, bf16_t);
-      else if (gated) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, float>), bf16_t, float);
-      else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, bf16_t>), bf16_t, bf16_t);
-      else KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, float>), bf16_t, float);
+      if (packed) {
+        if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, bf16_t, 1>), bf16_t, bf16_t);
+        else if (gated) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, float, 1>), bf16_t, float);
+        else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, bf16_t, 1>), bf16_t, bf16_t);
+        else KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, float, 1>), bf16_t, float);
+      } else {
+        if (gated && out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, bf16_t, 0>), bf16_t, bf16_t);
+        else if (gated) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<1, float, 0>), bf16_t, float);
+        else if (out_dtype == 1) KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, bf16_t, 0>), bf16_t, bf16_t);
+        else KVC_MOE_LAUNCH((moe_gemm_tiled_kernel<0, float, 0>), bf16_t, float);
+      }
     } else if (packed) {
       if (!vectors || N % 16 || K % 64)
         return kvc_fail("kvc_moe_gemm: a packed matrix has experts of a multiple of 16 rows of a multiple of 64");

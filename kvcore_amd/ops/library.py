@@ -1392,8 +1392,8 @@ def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: 
     if w.shape != (rows, K) or out.shape[0] < pairs or x.dtype != w.dtype or out.stride(1) != 1 or x.stride(1) != 1:
         raise KernelError("moe_gemm: shapes do not match")
     max_tiles = min(tiles.shape[0], moe_max_tiles(pairs, experts, tile_rows))
-    # single tokens stream the packed twin of the experts' matrix where the model keeps one
-    w_ptr, packed = (_streamed(w, N) if tile_rows == 16 and N % 16 == 0 and K % 64 == 0 else (_dev(w, "w"), 0))
+    # the bfloat16 kernels read the packed twin of the experts' matrix where the model keeps one
+    w_ptr, packed = (_streamed(w, N) if N % 16 == 0 and K % 64 == 0 else (_dev(w, "w"), 0))
     _check(load().kvc_moe_gemm(out.data_ptr(), out.stride(0), _code(out, "out"), x.data_ptr(), x.stride(0),
                                w_ptr, _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
                                _dev(tiles, "tiles", torch.int32), _dev(num_tiles, "num_tiles", torch.int32),
