@@ -370,7 +370,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
 }
 
 // bfloat16, tiles of 64 rows: a block of four waves takes the tile's rows and 128 columns (gated;
-// 256 otherwise).  The rows' chunk of 32 values along K goes through LDS, which all waves read as
+// 256 otherwise).  The rows' chunk of 64 values along K goes through LDS, which all waves read as
 // the B operand (four row blocks of 16); every wave fetches the weight rows of its own columns
 // straight into registers as the A operand (NF blocks of 16 columns, for gate and for up), one
 // chunk ahead of the products.  Every fetched weight meets 64 rows, every row 128 or 256 columns.
@@ -381,7 +381,8 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
   constexpr int NF = GATED ? 2 : 4;   // column blocks of 16 a wave
   constexpr int NR = kBigTileRows / 16;
-  constexpr int KROW = 40;            // a row's 32 values in LDS, padded against bank conflicts
+  constexpr int KC = 64;              // values of K a round (two matrix instructions deep)
+  constexpr int KROW = KC + 8;        // a row's chunk in LDS, padded against bank conflicts
   __shared__ __attribute__((aligned(16))) bf16_t x_s[kBigTileRows * KROW];
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;
@@ -390,12 +391,12 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
   const int li = lane & 15, lk = lane >> 4;
   const int n0 = (blockIdx.y * 4 + wave) * 16 * NF;
   const bool wave_live = n0 < N;  // the same for the whole wave
-  // staging: thread t brings 8 values of row t / 4 of the tile
+  // staging: thread t brings 16 values of row t / 4 of the tile
   const int srow = threadIdx.x >> 2, spart = threadIdx.x & 3;
   const bool srow_ok = srow < nr;
   const int srow_safe = srow_ok ? srow : 0;  // a row that is not there reads the tile's first, and is set to zero
   const int64_t in_row = in_div > 0 ? sorted[r0 + srow_safe] / in_div : r0 + srow_safe;
-  const bf16_t* xp = x + in_row * x_stride + 8 * spart;
+  const bf16_t* xp = x + in_row * x_stride + 16 * spart;
   const int64_t rows_per_expert = GATED ? 2 * static_cast<int64_t>(N) : N;
   const bf16_t* wp[NF];
 #pragma unroll
@@ -415,39 +416,58 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
       acc[f][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       if (GATED) acc2[f][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-  uint4 x_next = uint4{0u, 0u, 0u, 0u};
-  bf16x8_t w_next[NF], w2_next[GATED ? NF : 1];
+  uint4 x_next[2] = {uint4{0u, 0u, 0u, 0u}, uint4{0u, 0u, 0u, 0u}};
+  bf16x8_t w_next[2][NF], w2_next[2][GATED ? NF : 1];
+  // a round's second half may lie beyond K (K a multiple of 32 only): it then reads the first half
+  // again and is not multiplied
   auto fetch = [&](int k) {
-    x_next = *reinterpret_cast<const uint4*>(xp + k);
+    const bool two = k + 32 < K;
+    const int c0 = (two || spart < 2) ? 0 : -16 * spart;  // columns beyond K read the round's first instead
+    x_next[0] = *reinterpret_cast<const uint4*>(xp + k + c0);
+    x_next[1] = *reinterpret_cast<const uint4*>(xp + k + c0 + 8);
     if (wave_live) {
 #pragma unroll
-      for (int f = 0; f < NF; ++f) {
-        const int64_t wo = PACKED ? static_cast<int64_t>(k / 32) * 512 : k;
-        w_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + wo);
-        if (GATED) w2_next[f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + up_off + wo);
+      for (int h = 0; h < 2; ++h) {
+        const int kk = k + ((h && two) ? 32 : 0);
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          const int64_t wo = PACKED ? static_cast<int64_t>(kk / 32) * 512 : kk;
+          w_next[h][f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + wo);
+          if (GATED) w2_next[h][f] = *reinterpret_cast<const bf16x8_t*>(wp[f] + up_off + wo);
+        }
       }
     }
   };
   fetch(0);
-  for (int k = 0; k < K; k += 32) {
+  for (int k = 0; k < K; k += KC) {
+    const bool two = k + 32 < K;
     __syncthreads();  // the chunk before has been read by every wave
-    *reinterpret_cast<uint4*>(x_s + srow * KROW + 8 * spart) = srow_ok ? x_next : uint4{0u, 0u, 0u, 0u};
-    bf16x8_t wa[NF], wa2[GATED ? NF : 1];
+    // thread t's 16 values: columns 16 spart .. of the round; K shorter than a whole round leaves zeros
+    const bool keep = srow_ok && (two || spart < 2);
+    *reinterpret_cast<uint4*>(x_s + srow * KROW + 16 * spart) = keep ? x_next[0] : uint4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<uint4*>(x_s + srow * KROW + 16 * spart + 8) = keep ? x_next[1] : uint4{0u, 0u, 0u, 0u};
+    bf16x8_t wa[2][NF], wa2[2][GATED ? NF : 1];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      wa[f] = w_next[f];
-      if (GATED) wa2[f] = w2_next[f];
-    }
-    if (k + 32 < K) fetch(k + 32);
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        wa[h][f] = w_next[h][f];
+        if (GATED) wa2[h][f] = w2_next[h][f];
+      }
+    if (k + KC < K) fetch(k + KC);
     __syncthreads();
     if (wave_live) {  // scalar: matrix instructions are skipped by a branch, never by a lane mask
 #pragma unroll
-      for (int r = 0; r < NR; ++r) {
-        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(x_s + (16 * r + li) * KROW + 8 * lk);
+      for (int h = 0; h < 2; ++h) {
+        if (h == 1 && !two) break;  // scalar
 #pragma unroll
-        for (int f = 0; f < NF; ++f) {
-          acc[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[f], b, acc[f][r], 0, 0, 0);
-          if (GATED) acc2[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa2[f], b, acc2[f][r], 0, 0, 0);
+        for (int r = 0; r < NR; ++r) {
+          const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(x_s + (16 * r + li) * KROW + 32 * h + 8 * lk);
+#pragma unroll
+          for (int f = 0; f < NF; ++f) {
+            acc[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[h][f], b, acc[f][r], 0, 0, 0);
+            if (GATED) acc2[f][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa2[h][f], b, acc2[f][r], 0, 0, 0);
+          }
         }
       }
     }

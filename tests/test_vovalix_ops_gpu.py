@@ -408,11 +408,13 @@ def expert_weights(E, H, I, gen, shared=0):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("E,top,groups,keep,H,I,shared,T", [(6, 2, 3, 2, 96, 40, 56, 75), (8, 3, 1, 1, 128, 64, 0, 300),
                                                             (2, 2, 2, 2, 40, 8, 0, 1), (3, 1, 3, 1, 40, 16, 8, 2),
-                                                            (16, 4, 4, 1, 64, 32, 32, 33), (5, 2, 1, 1, 36, 20, 12, 19)])
+                                                            (16, 4, 4, 1, 64, 32, 32, 33), (5, 2, 1, 1, 36, 20, 12, 19),
+                                                            (4, 2, 1, 1, 96, 32, 0, 200), (2, 1, 1, 1, 160, 96, 16, 150)])
 def test_the_feed_forward_of_routed_experts(dtype, E, top, groups, keep, H, I, shared, T):
     """The part itself on rows of its own: routing, the arrangement by expert, both products,
     the weighted sum and the shared expert, against the plain function token by token.  Sizes
-    that 16-byte loads do not divide (36, 20, 12) take the kernel without them."""
+    that 16-byte loads do not divide (36, 20, 12) take the kernel without them; many rows an expert
+    take tiles of 64 rows (also with sums of 96, 160 and 32 terms, which end inside a round of 64)."""
     from kvcore_amd.engine.context import StepBuffers, StepContext
     from kvcore_amd.parts.base import Runtime
     from kvcore_amd.parts.moe import RoutedExperts
