@@ -99,7 +99,7 @@ def _vovalix_layers(n, width, heads, kv, experts, top, ff, groups, keep, chunk):
                  "mixer": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125,
                            "mask": {"size": chunk}}}
     gla = {"type": "gla", "mlp": moe,
-           "mixer": {"heads": heads // 2, "dim": 64, "vdim": 128, "tau": 16.0, "rank": 16}}
+           "mixer": {"heads": heads // 2, "dim": 64, "vdim": 128, "tau": 8.0, "rank": 32}}
     delta = {"type": "delta", "mlp": moe,
              "mixer": {"heads": heads // 2, "kv_heads": heads // 4, "dim": 128, "vdim": 128, "conv": 4}}
     return [(attention, gla, delta, gla)[i % 4] for i in range(n)]
@@ -252,7 +252,7 @@ def parse_args():
     p.add_argument("--dirulorn-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
                    help="with --dirulorn: run one of the workloads only (for profiling)")
     p.add_argument("--vovalix", default=None, choices=sorted(VOVALIX_SHAPES),
-                   help="instead of the contract's line: prefill and decode of a Vovalix shape beside the "
+                   help="instead of the headline line: prefill and decode of a Vovalix shape beside the "
                         "Dirulorn of the same width and depth; a line per model and workload")
     p.add_argument("--vovalix-only", default="both", choices=["both", "vovalix", "dirulorn"],
                    help="with --vovalix: run one of the two models only (for profiling)")

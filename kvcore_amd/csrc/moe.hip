@@ -262,12 +262,12 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(int32_t* __restrict__ s
   }
 }
 
-// bfloat16: a block of four waves takes one tile of rows and 64 columns (16 a wave).  A round covers
+// bfloat16: a block of four waves takes one tile of rows and 64 columns (16 a wave).  A pass covers
 // 64 values along K: lane (li, lk) fetches the 16 values from 16 lk of its weight row and of its
 // token row (32 contiguous bytes, so that the four lanes of a row read one 128-byte line) and the two
-// matrix instructions of the round take its first and its second eight (both operands are dealt the
-// same way, so each product still sums over all of K); the next two rounds' values are asked for
-// before this round's products.
+// matrix instructions of the pass take its first and its second eight (both operands are dealt the
+// same way, so each product still sums over all of K); the values of the next two passes are asked for
+// before this pass's products.
 template <int GATED, typename TO, int PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const bf16_t* wr2 = wr + static_cast<int64_t>(N) * K;  // the up rows follow the gate rows (in either order of storage)
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
   const int k_main = K & ~63;
-  // two rounds are on their way while one is multiplied
+  // two passes are on their way while one is multiplied
   bf16x8_t an[2][2], a2n[2][2], bn[2][2];
   auto fetch = [&](int k, int slot) {
 #pragma unroll
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   if (k_main > 0) fetch(0, 0);
   if (k_main > 64) fetch(64, 1);
   for (int k = 0; k < k_main; k += 128) {
-    // slot 0 holds round k, slot 1 round k + 64; each is asked for again as soon as it has been used
+    // slot 0 holds pass k, slot 1 pass k + 64; each is asked for again as soon as it has been used
     bf16x8_t a0[2], a20[2], b0[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
   constexpr int NF = GATED ? 2 : 4;   // column blocks of 16 a wave
   constexpr int NR = kBigTileRows / 16;
-  constexpr int KC = 64;              // values of K a round (two matrix instructions deep)
+  constexpr int KC = 64;              // values of K a pass (two matrix instructions deep)
   constexpr int KROW = KC + 8;        // a row's chunk in LDS, padded against bank conflicts
   __shared__ __attribute__((aligned(16))) bf16_t x_s[kBigTileRows * KROW];
   const int tile = blockIdx.x;
@@ -418,11 +418,11 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     }
   uint4 x_next[2] = {uint4{0u, 0u, 0u, 0u}, uint4{0u, 0u, 0u, 0u}};
   bf16x8_t w_next[2][NF], w2_next[2][GATED ? NF : 1];
-  // a round's second half may lie beyond K (K a multiple of 32 only): it then reads the first half
+  // a pass's second half may lie beyond K (K a multiple of 32 only): it then reads the first half
   // again and is not multiplied
   auto fetch = [&](int k) {
     const bool two = k + 32 < K;
-    const int c0 = (two || spart < 2) ? 0 : -16 * spart;  // columns beyond K read the round's first instead
+    const int c0 = (two || spart < 2) ? 0 : -16 * spart;  // columns beyond K read the pass's first instead
     x_next[0] = *reinterpret_cast<const uint4*>(xp + k + c0);
     x_next[1] = *reinterpret_cast<const uint4*>(xp + k + c0 + 8);
     if (wave_live) {
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
   for (int k = 0; k < K; k += KC) {
     const bool two = k + 32 < K;
     __syncthreads();  // the chunk before has been read by every wave
-    // thread t's 16 values: columns 16 spart .. of the round; K shorter than a whole round leaves zeros
+    // thread t's 16 values: columns 16 spart .. of the pass; K shorter than a whole pass leaves zeros
     const bool keep = srow_ok && (two || spart < 2);
     *reinterpret_cast<uint4*>(x_s + srow * KROW + 16 * spart) = keep ? x_next[0] : uint4{0u, 0u, 0u, 0u};
     *reinterpret_cast<uint4*>(x_s + srow * KROW + 16 * spart + 8) = keep ? x_next[1] : uint4{0u, 0u, 0u, 0u};

@@ -153,8 +153,8 @@ def test_small_kernels_around_the_recurrences():
     z = torch.randn(T, 48, generator=gen, dtype=torch.float64) * 6
     b = torch.randn(48, generator=gen, dtype=torch.float64)
     out = torch.empty(T, 48, device=DEV)
-    ops.sigmoid_power(out, gpu(z), gpu(b), 1 / 16.0)
-    assert rel(out, torch.sigmoid(z + b).pow(1 / 16.0)) < 1e-6
+    ops.sigmoid_power(out, gpu(z), gpu(b), 1 / 12.0)
+    assert rel(out, torch.sigmoid(z + b).pow(1 / 12.0)) < 1e-6
     # decay and write strength of the delta rule
     a_raw, b_raw = (torch.randn(T, 5, generator=gen, dtype=torch.float64) * 3 for _ in range(2))
     a_log, dt_bias = (torch.randn(5, generator=gen, dtype=torch.float64) for _ in range(2))
@@ -185,8 +185,8 @@ def test_small_kernels_around_the_recurrences():
     # the experts' activation
     gu = torch.randn(T, 2 * 24, generator=gen, dtype=torch.float64) * 3
     out = torch.empty(T, 24, device=DEV)
-    ops.clamped_glu(out, gpu(gu), 1.5, 1.702)
-    gg, uu = torch.clamp(gu[:, :24], max=1.5), torch.clamp(gu[:, 24:], -1.5, 1.5)
+    ops.clamped_glu(out, gpu(gu), 1.3, 1.702)
+    gg, uu = torch.clamp(gu[:, :24], max=1.3), torch.clamp(gu[:, 24:], -1.3, 1.3)
     assert rel(out, gg * torch.sigmoid(1.702 * gg) * (uu + 1)) < 1e-6
 
 
@@ -336,7 +336,7 @@ def test_matrix_core_kernels_with_bias_and_chunks(kernel, H, G, d, chunk):
 
 # --------------------------------------------------------------------- routed experts
 @pytest.mark.parametrize("E,top,groups,keep", [(6, 2, 3, 2), (8, 3, 1, 1), (2, 2, 2, 2), (3, 1, 3, 1), (16, 4, 4, 1),
-                                               (16, 4, 4, 2), (12, 4, 3, 2), (5, 5, 1, 1), (70, 6, 10, 3)])
+                                               (16, 4, 4, 2), (12, 3, 4, 3), (5, 5, 1, 1), (70, 6, 10, 3)])
 def test_routing_against_the_plain_rule(E, top, groups, keep):
     from kvcore_amd.ops import library as ops
 
@@ -414,7 +414,7 @@ def test_the_feed_forward_of_routed_experts(dtype, E, top, groups, keep, H, I, s
     """The part itself on rows of its own: routing, the arrangement by expert, both products,
     the weighted sum and the shared expert, against the plain function token by token.  Sizes
     that 16-byte loads do not divide (36, 20, 12) take the kernel without them; many rows an expert
-    take tiles of 64 rows (also with sums of 96, 160 and 32 terms, which end inside a round of 64)."""
+    take tiles of 64 rows (also with sums of 96, 160 and 32 terms, which end inside a pass of 64)."""
     from kvcore_amd.engine.context import StepBuffers, StepContext
     from kvcore_amd.parts.base import Runtime
     from kvcore_amd.parts.moe import RoutedExperts

@@ -62,10 +62,10 @@ CONFIG_A = {
 CONFIG_B = {
     "architecture": "Vovalix", "vocab": 320, "width": 128, "norm": {"eps": 1e-6}, "logit_scale": 0.5,
     "layers": [
-        {"type": "delta", "mixer": _delta(2, 2, 64, 64, 4), "mlp": _moe(8, 3, 64, 1.5)},
-        {"type": "attention", "mixer": _attn(8, 2, 64, 64, 0.125, 48), "mlp": _moe(8, 3, 64, 1.5)},
-        {"type": "gla", "mixer": _gla(2, 64, 64, 16.0, 16), "mlp": _moe(4, 1, 128, 3.0, groups=(2, 1), shared=(64, 1.0))},
-        {"type": "attention", "mixer": _attn(8, 2, 64, 64, 0.125, 48), "mlp": _moe(8, 3, 64, 1.5), "weights_of": 1},
+        {"type": "delta", "mixer": _delta(2, 2, 64, 64, 4), "mlp": _moe(8, 3, 64, 2.0)},
+        {"type": "attention", "mixer": _attn(8, 2, 64, 64, 0.125, 48), "mlp": _moe(8, 3, 64, 2.0)},
+        {"type": "gla", "mixer": _gla(2, 64, 64, 12.0, 24), "mlp": _moe(4, 1, 128, 3.0, groups=(2, 1), shared=(64, 1.0))},
+        {"type": "attention", "mixer": _attn(8, 2, 64, 64, 0.125, 48), "mlp": _moe(8, 3, 64, 2.0), "weights_of": 1},
     ],
 }
 
