@@ -217,6 +217,38 @@ def test_the_stream_after_every_layer_run(models, dtype):
         assert err < limit, f"layer run {i}: {err:.3e}"
 
 
+@pytest.mark.parametrize("seed", [0, 6, 9, 21, 23, 27, 34, 56])
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Models whose every size, constant and layer order is drawn from a seed (widths that 8 does not
+    divide, values wider than keys, chunks of 7 to 128 positions, one to twelve experts, borrowed
+    layers, layers without a feed-forward), in float32, where the engine and the plain model agree
+    to rounding whatever the routers choose: two requests side by side, portions, then single tokens."""
+    import random
+
+    from tests.vovalix_helpers import random_config
+
+    cfg = random_config(random.Random(seed))
+    folder = make_model_dir(tmp_path / "drawn", cfg, seed=seed)
+    c, w = plain.load_model_folder(folder)
+    seqs = {"a": random_tokens(150, cfg["vocab"], seed + 1), "b": random_tokens(70, cfg["vocab"], seed + 2)}
+    want = {k: plain.vovalix_forward(c, w, v) for k, v in seqs.items()}
+    s = session_for(folder, torch.float32, 16, 320, max_num_seqs=4)
+    at = {"a": 0, "b": 0}
+    steps = []
+    for who, count in [("a", 37), ("b", 2), ("a", 50), ("b", 33)] + [("ab", 1)] * 30 + [("a", 33), ("b", 5)]:
+        entries = []
+        for k in who:
+            lo, hi = at[k], min(at[k] + count, len(seqs[k]))
+            if hi > lo:
+                entries.append({"id": k, "tokens": seqs[k][lo:hi], "want": list(range(hi - lo))})
+                at[k] = hi
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": [k for k in who if at[k] == len(seqs[k])]})
+    got = collect(s, steps)
+    assert len(got) == 220
+    compare(got, want, torch.float32)
+
+
 def test_attention_with_a_bias_and_chunks_runs_where_it_is_meant_to(models):
     """In bfloat16 with keys and values of 64 the chunked, biased attention takes the matrix-core
     kernels (portions and single tokens); in float32 the general kernel."""

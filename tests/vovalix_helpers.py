@@ -97,6 +97,50 @@ CONFIG_D = {
 CONFIGS = {"A": (CONFIG_A, 8), "B": (CONFIG_B, 16), "C": (CONFIG_C, 4), "D": (CONFIG_D, 16)}
 
 
+def random_config(rng) -> dict:
+    """A configuration drawn from ``rng`` (a ``random.Random``): three to eight layers of any kind in any
+    order, some borrowing an earlier layer's tensors, some without a feed-forward; widths, head counts
+    and grouping, key and value sizes, chunks, taps, ranks, experts, groups and choices all drawn anew."""
+    width = rng.choice([64, 96, 128, 192, 256, 320, 100])
+    def moe():
+        groups = rng.choice([1, 2, 3, 4])
+        per = rng.choice([1, 2, 3, 4])
+        E = groups * per
+        keep = rng.randint(1, groups)
+        top = rng.randint(1, min(4, keep * per))
+        m = {"kind": "moe", "expert": {"ff": rng.choice([24, 32, 48, 64, 96, 40]), "limit": rng.choice([0.5, 1.0, 2.5])},
+             "router": {"experts": E, "top": top}}
+        if groups > 1 or rng.random() < 0.5:  # a single group may also go unsaid
+            m["router"]["groups"] = {"count": groups, "keep": keep}
+        if rng.random() < 0.6: m["shared"] = {"ff": rng.choice([16, 64, 128, 72]), "limit": rng.choice([0.7, 1.5])}
+        return m
+    def attn():
+        kv = rng.choice([1, 2, 3, 4]); g = rng.choice([1, 2, 4])
+        dim = rng.choice([16, 32, 48, 64, 64, 128]); vdim = rng.choice([dim, dim, 2 * dim if dim <= 64 else dim, 24, 80])
+        m = {"heads": kv * g, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": rng.choice([0.125, 0.2, 0.09])}
+        if rng.random() < 0.85: m["mask"] = {"size": rng.choice([7, 16, 33, 64, 100, 128, 50])}
+        return m
+    def gla():
+        return {"heads": rng.choice([1, 2, 3, 6]), "dim": rng.choice([8, 16, 32, 48, 64, 20]), "vdim": rng.choice([16, 64, 32, 40, 128]),
+                "tau": rng.choice([4.0, 16.0, 7.5]), "rank": rng.choice([4, 8, 16, 5])}
+    def delta():
+        kv = rng.choice([1, 2, 3]); g = rng.choice([1, 2])
+        return {"heads": kv * g, "kv_heads": kv, "dim": rng.choice([16, 32, 64, 128, 24]), "vdim": rng.choice([16, 32, 64, 128, 40]),
+                "conv": rng.choice([1, 2, 3, 4])}
+    kinds = {"attention": attn, "gla": gla, "delta": delta}
+    layers = []
+    for i in range(rng.randint(3, 8)):
+        own = [j for j, l in enumerate(layers) if "weights_of" not in l]
+        if own and rng.random() < 0.3:
+            j = rng.choice(own)
+            l = dict(layers[j]); l["weights_of"] = j
+            layers.append(l); continue
+        t = rng.choice(list(kinds))
+        layers.append({"type": t, "mixer": kinds[t](), "mlp": moe() if rng.random() < 0.85 else None})
+    return {"architecture": "Vovalix", "vocab": rng.choice([97, 256, 512, 1000]), "width": width,
+            "norm": {"eps": rng.choice([1e-6, 1e-5])}, "logit_scale": rng.choice([1.0, 2.0, 0.5]), "layers": layers}
+
+
 def make_model_dir(folder: Path, config: dict, seed: int) -> Path:
     """A model folder from the product's random-weights mode, with the small tensors redrawn so
     that each one matters: biases and decay parameters get values that spread the decays between
