@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
   }
   // one stage's tokens, from the LDS buffers given
   auto work_stage = [&](const float* q_s, const float* k_s, const float* a_s, const float* v_s, int t0, int nt) {
-    for (int tt = 0; tt < nt; ++tt) {
+    auto token = [&](int tt) {
       const float* qt = q_s + tt * d + (FULL ? ns * NPT : ns);
       const float* kt = k_s + tt * d + (FULL ? ns * NPT : ns);
       constexpr int ST = FULL ? 1 : NSL;  // from one of the thread's rows to its next, in LDS
@@ -164,6 +164,14 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       }
       acc = group_sum<NSL>(acc);
       if (ns == 0 && c_ok) out[static_cast<int64_t>(t0 + tt) * width + h * dv + c] = acc;
+    };
+    if (nt == LSC) {
+      // a whole stage: unrolled, so that a token's LDS reads are under way while the token before
+      // it is still being worked on (only the state itself passes from token to token)
+#pragma unroll 4
+      for (int tt = 0; tt < LSC; ++tt) token(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) token(tt);
     }
   };
   if constexpr (PF) {
