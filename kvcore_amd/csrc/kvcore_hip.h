@@ -227,9 +227,10 @@ int kvc_sigmoid_power(float* a, const float* z, int64_t z_stride, const float* b
 int kvc_decay_and_write_gates(float* g, float* beta, const float* a_raw, int64_t a_stride,
                               const float* b_raw, int64_t b_stride, const float* a_log,
                               const float* dt_bias, int T, int nh, kvc_stream stream);
-// x[t, h, :] *= scale / sqrt(sum x[t, h, :]^2 + eps), in place, heads of d float32 values.
+// x[t, h, :] *= scale / sqrt(sum x[t, h, :]^2 + eps), in place, heads of d float32 values; the first
+// first_heads heads take first_scale instead of scale.
 int kvc_unit_heads(float* x, int64_t stride, int T, int heads, int d, float eps, float scale,
-                   kvc_stream stream);
+                   int first_heads, float first_scale, kvc_stream stream);
 // out[t, h, c] = o[t, h, c] / sqrt(mean_c o[t, h, :]^2 + eps) * gain[c] * silu(gate[t, h, c]).
 int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* gate,
                           int64_t gate_stride, int gate_dtype, const float* gain, float eps, int T,
@@ -260,8 +261,9 @@ int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, in
                  int gated, float limit, float alpha, int packed, kvc_stream stream);
 // out[t] = sum_c weight[t, c] * y[t * top + c] + add0[t] + add1[t] (either may be null; add0 of
 // dtype add0_dtype, add1 float32), float32.
+// accumulate: the sum is added into out instead of stored.
 int kvc_moe_combine(float* out, const float* y, const float* weight, int top, const void* add0,
-                    int add0_dtype, const float* add1, int T, int H, kvc_stream stream);
+                    int add0_dtype, const float* add1, int T, int H, int accumulate, kvc_stream stream);
 // out[t, i] = g * sigmoid(alpha * g) * (u + 1), g = min(gate_up[t, i], limit),
 // u = clamp(gate_up[t, I + i], -limit, limit).
 int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, float limit, float alpha, int dtype,

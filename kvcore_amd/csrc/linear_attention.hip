@@ -298,10 +298,11 @@ __global__ __launch_bounds__(256) void decay_and_write_gates_kernel(
   beta[idx] = sigmoid_f(b_raw[t * b_stride + h]);
 }
 
-// Heads of d float32 values made unit vectors in place, x / sqrt(sum x^2 + eps) * scale: a wave a
-// (token, head).
+// Heads of d float32 values made unit vectors in place, x / sqrt(sum x^2 + eps) * scale (the first
+// first_heads heads times first_scale instead): a wave a (token, head).
 __global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, int64_t stride, int T, int heads,
-                                                         int d, float eps, float scale) {
+                                                         int d, float eps, float scale, int first_heads,
+                                                         float first_scale) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (item >= static_cast<int64_t>(T) * heads) return;
@@ -310,7 +311,7 @@ __global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, 
   float ss = 0.f;
   for (int i = lane; i < d; i += kWave) ss = fmaf(p[i], p[i], ss);
   ss = wave_sum(ss);
-  const float inv = scale / sqrtf(ss + eps);
+  const float inv = (h < first_heads ? first_scale : scale) / sqrtf(ss + eps);
   for (int i = lane; i < d; i += kWave) p[i] *= inv;
 }
 
@@ -431,13 +432,13 @@ extern "C" int kvc_decay_and_write_gates(float* g, float* beta, const float* a_r
 }
 
 extern "C" int kvc_unit_heads(float* x, int64_t stride, int T, int heads, int d, float eps, float scale,
-                              kvc_stream stream) {
+                              int first_heads, float first_scale, kvc_stream stream) {
   if (T < 0 || heads <= 0 || d <= 0 || stride < static_cast<int64_t>(heads) * d)
     return kvc_fail("kvc_unit_heads: bad sizes");
   if (T == 0) return 0;
   const int64_t waves = static_cast<int64_t>(T) * heads;
   hipLaunchKernelGGL(unit_heads_kernel, dim3(static_cast<unsigned>((waves + 3) / 4)), dim3(256), 0, S(stream), x,
-                     stride, T, heads, d, eps, scale);
+                     stride, T, heads, d, eps, scale, first_heads, first_scale);
   return kvc_check_launch("kvc_unit_heads");
 }
 

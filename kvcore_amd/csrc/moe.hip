@@ -19,7 +19,7 @@
 //                    the A operand, the tokens as B) with float32 sums; float32 operands, and rows
 //                    that 16-byte loads do not divide, are summed in float32 in index order.  A row's sums do not depend on which tile it is in.
 //   kvc_moe_combine  out[t] = sum_c weight[t, c] * y[t * top + c] (+ up to two more row sets),
-//                    float32, in the order of the choices.
+//                    float32, in the order of the choices; or added into out (the residual stream).
 //   kvc_clamped_glu  the same activation for a feed-forward that every token runs.
 
 #include <hip/hip_runtime.h>
@@ -525,7 +525,7 @@ template <typename TA>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
                                                           const float* __restrict__ weight, int top,
                                                           const TA* __restrict__ add0, const float* __restrict__ add1,
-                                                          int T, int H) {
+                                                          int T, int H, int accumulate) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= static_cast<int64_t>(T) * H) return;
   const int t = static_cast<int>(idx / H), c = static_cast<int>(idx - static_cast<int64_t>(t) * H);
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ ou
     acc = fmaf(weight[static_cast<int64_t>(t) * top + j], y[(static_cast<int64_t>(t) * top + j) * H + c], acc);
   if (add0 != nullptr) acc += to_float(add0[idx]);
   if (add1 != nullptr) acc += add1[idx];
-  out[idx] = acc;
+  out[idx] = accumulate ? out[idx] + acc : acc;
 }
 
 template <typename T>
@@ -683,17 +683,18 @@ extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const 
 }
 
 extern "C" int kvc_moe_combine(float* out, const float* y, const float* weight, int top, const void* add0,
-                               int add0_dtype, const float* add1, int T, int H, kvc_stream stream) {
+                               int add0_dtype, const float* add1, int T, int H, int accumulate,
+                               kvc_stream stream) {
   if (T < 0 || H <= 0 || top < 0) return kvc_fail("kvc_moe_combine: bad sizes");
   if (T == 0) return 0;
   const int64_t n = static_cast<int64_t>(T) * H;
   const dim3 grid(static_cast<unsigned>((n + 255) / 256));
   if (add0_dtype == 1) {
     hipLaunchKernelGGL((moe_combine_kernel<bf16_t>), grid, dim3(256), 0, S(stream), out, y, weight, top,
-                       static_cast<const bf16_t*>(add0), add1, T, H);
+                       static_cast<const bf16_t*>(add0), add1, T, H, accumulate);
   } else {
     hipLaunchKernelGGL((moe_combine_kernel<float>), grid, dim3(256), 0, S(stream), out, y, weight, top,
-                       static_cast<const float*>(add0), add1, T, H);
+                       static_cast<const float*>(add0), add1, T, H, accumulate);
   }
   return kvc_check_launch("kvc_moe_combine");
 }

@@ -51,7 +51,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, P],
         "kvc_sigmoid_power": [P, P, L, P, F, I, I, P],
         "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
-        "kvc_unit_heads": [P, L, I, I, I, F, F, P],
+        "kvc_unit_heads": [P, L, I, I, I, F, F, I, F, P],
         "kvc_head_rmsnorm_gate": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_moe_route": [P, P, P, I, I, I, I, I, P],
         "kvc_moe_router": [P, P, P, L, I, P, I, I, I, I, I, I, P],
@@ -59,7 +59,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_moe_tile_rows": [I, I],
         "kvc_moe_align": [P, P, P, P, I, I, I, I, P],
         "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
-        "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, P],
+        "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, I, P],
         "kvc_clamped_glu": [P, P, I, I, F, F, I, P],
         "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_add_layernorm": [P, P, P, P, P, F, I, I, I, P],
@@ -1308,12 +1308,14 @@ def decay_and_write_gates(g: torch.Tensor, beta: torch.Tensor, a_raw: torch.Tens
            "kvc_decay_and_write_gates")
 
 
-def unit_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0) -> None:
+def unit_heads(x: torch.Tensor, heads: int, dim: int, eps: float, scale: float = 1.0, first_heads: int = 0,
+               first_scale: float = 1.0) -> None:
     """Every head of ``dim`` values of the float32 rows ``x [T, heads * dim]`` (a column view is
-    fine) over its Euclidean length (``eps`` inside the root), times ``scale``, in place."""
+    fine) over its Euclidean length (``eps`` inside the root), times ``scale`` (the first
+    ``first_heads`` heads times ``first_scale`` instead), in place."""
     xp, xs = _f32_rows(x, "x", heads * dim)
-    _check(load().kvc_unit_heads(xp, xs, x.shape[0], heads, dim, float(eps), float(scale), _stream()),
-           "kvc_unit_heads")
+    _check(load().kvc_unit_heads(xp, xs, x.shape[0], heads, dim, float(eps), float(scale), int(first_heads),
+                                 float(first_scale), _stream()), "kvc_unit_heads")
 
 
 def head_rmsnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps: float,
@@ -1402,9 +1404,9 @@ def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: 
 
 
 def moe_combine(out: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, add0: torch.Tensor | None = None,
-                add1: torch.Tensor | None = None) -> None:
+                add1: torch.Tensor | None = None, accumulate: bool = False) -> None:
     """``out[t] = sum_c weight[t, c] * y[t * top + c] (+ add0[t]) (+ add1[t])``, float32; ``add0``
-    of either dtype, ``add1`` float32."""
+    of either dtype, ``add1`` float32.  ``accumulate``: the sum is added into ``out``."""
     T, H = out.shape
     top = weight.shape[1] if weight.dim() == 2 else 0
     if out.dtype != torch.float32 or (top and (y.shape[0] < T * top or y.shape[1] != H)):
@@ -1415,8 +1417,8 @@ def moe_combine(out: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, add0: 
     _check(load().kvc_moe_combine(_dev(out, "out"), _dev(y, "y", torch.float32), _dev(weight, "weight", torch.float32),
                                   top, None if add0 is None else _dev(add0, "add0"),
                                   0 if add0 is None else _code(add0, "add0"),
-                                  None if add1 is None else _dev(add1, "add1", torch.float32), T, H, _stream()),
-           "kvc_moe_combine")
+                                  None if add1 is None else _dev(add1, "add1", torch.float32), T, H,
+                                  int(bool(accumulate)), _stream()), "kvc_moe_combine")
 
 
 def clamped_glu(out: torch.Tensor, gate_up: torch.Tensor, limit: float, alpha: float) -> None:

@@ -130,6 +130,9 @@ class ParallelResidualBlock(Block):
         a = self.mixer.forward(x, ctx, call)
         if self.mixer_only:
             ops.residual_add(residual, a)
+        elif a.dtype == torch.float32 and hasattr(self.ffn, "forward_into"):
+            # a feed-forward whose last kernel can add into the stream takes the mixer's rows along
+            self.ffn.forward_into(residual, x, ctx, call, add=a)
         else:
             f = self.ffn.forward(x, ctx, call)
             ops.residual_add2(residual, a, f)

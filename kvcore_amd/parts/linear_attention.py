@@ -179,8 +179,9 @@ class GatedDeltaRule(_MatrixStateMixer):
         qkv = ctx.buf(f"gdr_qkv:{self.conv_dim}", self.conv_dim, torch.float32)
         ops.causal_conv(qkv, proj[:, : self.conv_dim], p["conv.weight"], None, conv_state, act="silu",
                         single_tokens=ctx.max_query_len == 1, **batch)
-        ops.unit_heads(qkv[:, :qk], self.qk_heads, self.dim, self.unit_eps, self.q_scale)
-        ops.unit_heads(qkv[:, qk:2 * qk], self.qk_heads, self.dim, self.unit_eps, 1.0)
+        # q and k in one launch: the q heads come first and take their scale
+        ops.unit_heads(qkv[:, :2 * qk], 2 * self.qk_heads, self.dim, self.unit_eps, 1.0,
+                       first_heads=self.qk_heads, first_scale=self.q_scale)
         g = ctx.buf(f"gdr_g:{nh}", nh, torch.float32)
         beta = ctx.buf(f"gdr_beta:{nh}", nh, torch.float32)
         at = self.conv_dim + inner

@@ -72,7 +72,12 @@ class RoutedExperts(FeedForward):
         shared = ("shared.gate_up", "shared.down") if self.shared_size else ()
         return ("experts.gate_up", "experts.down", *shared)
 
-    def forward(self, x, ctx, call, sink=None):
+    def forward_into(self, residual, x, ctx, call, add=None):
+        """``residual += add + ff(x)`` (float32 rows), the sums made in the kernel that adds up the
+        experts: what a block calls that would otherwise add the result into the stream itself."""
+        self.forward(x, ctx, call, into=residual, add=add)
+
+    def forward(self, x, ctx, call, sink=None, into=None, add=None):
         p, H, E, I, top = self.params, self.hidden_size, self.experts, self.expert_size, self.top
         T = ctx.num_tokens
         pairs = T * top
@@ -104,6 +109,9 @@ class RoutedExperts(FeedForward):
             ops.clamped_glu(sact, gate_up, self.shared_limit, self.alpha)
             shared = ctx.buf(f"moe_shared_out:{H}", H, torch.float32)
             ops.linear(shared, sact, p["shared.down"])
+        if into is not None:
+            ops.moe_combine(into, y, weight, shared, add, accumulate=True)
+            return into
         out = ctx.buf("ffn_out_f32", H, torch.float32)
         ops.moe_combine(out, y, weight, shared, None)
         return out

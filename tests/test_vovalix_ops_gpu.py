@@ -169,6 +169,12 @@ def test_small_kernels_around_the_recurrences():
     ops.unit_heads(xg[:, :72], 3, 24, 1e-6, 24 ** -0.5)
     want = plain.unit_vector(x[:, :72].reshape(T, 3, 24)).reshape(T, 72) * 24 ** -0.5
     assert rel(xg[:, :72], want) < 1e-6 and torch.equal(xg[:, 72:].cpu().double(), x[:, 72:].float().double())
+    # the first heads with a scale of their own (q before k in one launch)
+    xg = gpu(x)
+    ops.unit_heads(xg[:, :72], 3, 24, 1e-6, 1.0, first_heads=1, first_scale=0.25)
+    want = plain.unit_vector(x[:, :72].reshape(T, 3, 24))
+    want[:, 0] *= 0.25
+    assert rel(xg[:, :72], want.reshape(T, 72)) < 1e-6
     # the head norm with its gate, heads of 40 and of 1 and of 130 values
     for heads, dv in ((3, 40), (4, 1), (2, 130)):
         o = torch.randn(T, heads, dv, generator=gen, dtype=torch.float64)
@@ -449,7 +455,15 @@ def test_the_feed_forward_of_routed_experts(dtype, E, top, groups, keep, H, I, s
     out = part.forward(gpu(x, dtype), ctx, None)
     assert out.dtype == torch.float32 and out.shape == (T, H)
     assert rel(out, want) < (3e-6 if dtype == torch.float32 else 8e-3)
+    # the form that adds into a stream, with another branch's rows taken along
+    stream = torch.randn(T, H, generator=gen, dtype=torch.float64)
+    other = torch.randn(T, H, generator=gen, dtype=torch.float64)
+    first = out.double().cpu().clone()
+    stream_gpu = gpu(stream)
+    part.forward_into(stream_gpu, gpu(x, dtype), ctx, None, add=gpu(other))
+    assert rel(stream_gpu, stream.float().double() + (other.float().double() + first)) < 1e-6
     # the same rows again among others, in another order: a row's result does not depend on its place
+    out = part.forward(gpu(x, dtype), ctx, None)
     if T > 2:
         first = out.cpu().clone()  # the result lives in a step buffer that the next call rewrites
         perm = torch.randperm(T, generator=gen)
