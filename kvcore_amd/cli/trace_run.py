@@ -61,9 +61,19 @@ def main(argv=None) -> int:
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
-    session = TraceSession(args.model, dtype, max_tokens=args.max_tokens, block_size=args.block_size,
-                           max_num_seqs=args.max_num_seqs, device=args.device,
-                           poison_cache=args.poison_cache, shuffle_pages=args.shuffle_pages)
+    # a pool so large that a request's block table would outgrow what a kernel serves takes larger
+    # pages (the parts refuse the smaller ones when the runner is built, with a message that says so)
+    session, block_size = None, args.block_size
+    while session is None:
+        try:
+            session = TraceSession(args.model, dtype, max_tokens=args.max_tokens, block_size=block_size,
+                                   max_num_seqs=args.max_num_seqs, device=args.device,
+                                   poison_cache=args.poison_cache, shuffle_pages=args.shuffle_pages)
+        except ValueError as exc:
+            if "block_size" not in str(exc) or block_size >= 256:
+                raise
+            block_size *= 2
+            print(f"trace_run: pages of {block_size} tokens ({exc})", file=sys.stderr, flush=True)
     print("trace_run: ready", file=sys.stderr, flush=True)
 
     for line in sys.stdin:
