@@ -415,7 +415,8 @@ def expert_weights(E, H, I, gen, shared=0):
 @pytest.mark.parametrize("E,top,groups,keep,H,I,shared,T", [(6, 2, 3, 2, 96, 40, 56, 75), (8, 3, 1, 1, 128, 64, 0, 300),
                                                             (2, 2, 2, 2, 40, 8, 0, 1), (3, 1, 3, 1, 40, 16, 8, 2),
                                                             (16, 4, 4, 1, 64, 32, 32, 33), (5, 2, 1, 1, 36, 20, 12, 19),
-                                                            (4, 2, 1, 1, 96, 32, 0, 200), (2, 1, 1, 1, 160, 96, 16, 150)])
+                                                            (4, 2, 1, 1, 96, 32, 0, 200), (2, 1, 1, 1, 160, 96, 16, 150),
+                                                            (2, 2, 2, 2, 64, 32, 0, 300), (3, 1, 1, 1, 96, 64, 24, 800)])
 def test_the_feed_forward_of_routed_experts(dtype, E, top, groups, keep, H, I, shared, T):
     """The part itself on rows of its own: routing, the arrangement by expert, both products,
     the weighted sum and the shared expert, against the plain function token by token.  Sizes
